@@ -939,6 +939,83 @@ const char *vmx_gguf_metadata_string(const vmx_gguf *g, const char *key, int arr
 /* "model.layers.3.self_attn.q_proj" -> "blk.3.attn_q"; candidate `which` in priority order; returns the length, 0 if none */
 int vmx_gguf_llama_cpp_name(const char *hf_prefix, int which, char *out, size_t out_bytes);
 
+/* ------------------------------------------------- latent attention, grouped router, Gesutar executor */
+
+/* Latent attention (compressed keys/values): a token's cache row is [c | k_rot] with c the RMS-normed latent (kv_rank values)
+ * and k_rot one rotated key part (rot_dim values) shared by all heads.
+ * vmx_latent_kv_prepare: from the f32 rows `fused` [tokens, ld_fused] holding the query projection at column q_offset (per
+ * head [dim unrotated | rot_dim rotated]) and the down-projection at column dkv_offset ([kv_rank | rot_dim]):
+ * c = x / sqrt(mean(x^2) + eps) * latent_norm_w and the rotated key part go to cache row slots[t] (negative slot: not stored),
+ * the heads' rotated query parts to q_rot f32 [tokens, heads, rot_dim].  Rotation: interleaved pairs (2i, 2i + 1) of the first
+ * rot_dims dimensions by the angle positions[t] * inv_freq[i] (f32); later dimensions pass unchanged.  cache_dtype VMX_F32 / VMX_BF16. */
+int vmx_latent_kv_prepare(const float *fused, int64_t ld_fused, int q_offset, int dkv_offset, const uint16_t *latent_norm_w, float eps,
+                          const float *inv_freq, int rot_dims, const int32_t *positions, const int32_t *slots, void *cache,
+                          int cache_dtype, float *q_rot, int tokens, int heads, int dim, int rot_dim, int kv_rank, void *stream);
+/* vmx_latent_attention: out_latent[t, h] = sum_j p_j c_j over the keys j of sequence seq_ids[t] with 0 <= positions[t] - j < window
+ * (window 0: every earlier key), p = softmax((q_abs[t, h] . c_j + q_rot[t, h] . k_rot_j) * scale) whose denominator also holds
+ * exp(sink_bf16[h]) when sink_bf16 is given (a key-less, unscaled term).  q_abs is the query mapped into the latent space
+ * (U_h^T q_h); the caller maps out_latent through the value up-projection.  Cache rows are found through block_tables
+ * [sequences, max_blocks_per_seq] (row = block * block_size + position % block_size).  All f32 except the cache (VMX_F32 / VMX_BF16). */
+int vmx_latent_attention(float *out_latent, const float *q_abs, const float *q_rot, const void *cache, int cache_dtype,
+                         const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
+                         const uint16_t *sink_bf16, float scale, int window, int tokens, int heads, int kv_rank, int rot_dim,
+                         int block_size, void *stream);
+
+/* Router with group-limited selection: softmax over all experts (f32 logits [tokens, num_experts <= 256]); the experts form
+ * `groups` equal runs of neighbours, a group's score is its largest probability, only experts of the keep_groups best groups can
+ * be chosen; k rounds of argmax (ties -> smaller index).  weights = chosen probabilities / (their sum + 1e-20) * scale. */
+int vmx_grouped_topk_router(const float *logits, float *topk_weights, int32_t *topk_ids, int tokens, int num_experts, int k,
+                            int groups, int keep_groups, float scale, void *stream);
+
+/* y [M, N] = x [M, K] @ W [N, K]^T over bf16 weights, any shape; x and y in f32 (dtype VMX_F32) or bf16 (VMX_BF16).
+ * exact != 0: true f32 products on the vector ALU; else bf16 operands on the matrix cores where the shape allows.  f32 accumulation. */
+int vmx_linear_bf16w(void *y, int y_dtype, const void *x, int x_dtype, const uint16_t *w, int M, int N, int K, int exact, void *stream);
+
+#define VMX_MIXER_LATENT_ATTENTION 0
+#define VMX_MLP_NONE 0
+#define VMX_MLP_MOE 1
+
+/* One layer of a Gesutar model: the mixer's sizes and constants, then the feed-forward's. */
+typedef struct vmx_gesutar_layer_config {
+    int mixer;                 /* VMX_MIXER_* */
+    int heads, dim, rot_dim, vdim, kv_rank;   /* per head: dim unrotated + rot_dim rotated query/key dimensions, vdim values; latent size */
+    int window;                /* position i sees j with 0 <= i - j < window */
+    int rot_dims;              /* rotated dimensions (<= rot_dim, even) */
+    double rot_base;           /* inv_freq[i] = rot_base^(-2 i / rot_dims) */
+    float scale;               /* score scale */
+    int mlp;                   /* VMX_MLP_* */
+    int experts, top, groups, keep_groups, expert_ff, shared_ff;   /* shared_ff 0: no shared expert */
+    float router_scale;
+} vmx_gesutar_layer_config;
+
+typedef struct vmx_gesutar_config {
+    int vocab, width, num_layers;
+    float norm_eps;
+    double embed_scale;
+    int bigram_buckets, bigram_mul_prev, bigram_mul_cur;   /* buckets 0: no bigram table */
+    int dtype;                 /* VMX_BF16: bf16 operands and cache; VMX_F32: everything in f32 */
+    int block_size, num_blocks;   /* paged cache: rows per block, blocks per layer */
+    int max_tokens, max_seqs;  /* most tokens / sequences of one forward call */
+} vmx_gesutar_config;
+
+typedef struct vmx_gesutar vmx_gesutar;
+int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesutar_layer_config *layers, vmx_gesutar **out);
+void vmx_gesutar_destroy(vmx_gesutar *m);
+/* One checkpoint tensor under its name in the file ("embed", "bigram", "head", "final.norm", "l<i>.norm1|norm2",
+ * "l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o", "l<i>.mlp.router", "l<i>.mlp.e<j>.up|down", "l<i>.mlp.shared.up|down"): bf16,
+ * matrices [out, in]; host or device memory; synchronises the stream. */
+int vmx_gesutar_load_tensor(vmx_gesutar *m, const char *name, const void *data, size_t bytes, void *stream);
+int vmx_gesutar_missing_tensors(const vmx_gesutar *m);   /* tensors still to load; vmx_last_error() names the first */
+/* One step over packed tokens (all arrays device i32): token t has id tokens[t], previous id prev_tokens[t] (-1: first token of
+ * its sequence), position positions[t], cache row slots[t], and belongs to sequence seq_ids[t] whose blocks are
+ * block_tables[seq_ids[t]].  Prompts, prompt portions and decode tokens may share a step; the new tokens' cache rows are
+ * written before attention reads them.  logits f32 [num_logit_rows, vocab] for the token rows logit_rows (optional), greedy_ids
+ * their argmax (optional), layer_trace f32 [layers, tokens, width] the residual stream after every layer (optional). */
+int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const int32_t *prev_tokens, const int32_t *positions, const int32_t *slots,
+                        const int32_t *seq_ids, int num_tokens, const int32_t *block_tables, int num_seqs, int max_blocks_per_seq,
+                        const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids, float *layer_trace,
+                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -211,6 +211,15 @@ _SIGS = {
     "vmx_gemma4_kv_scales_reset": (_i, [_p, _f, _p]),
     "vmx_gemma4_kv_scales_get": (_i, [_p, _i, _p, _p, _p, _p]),
     "vmx_gemma4_debug_kv": (_i, [_p, _i, _i, _i, _p, _sz, _p]),
+    "vmx_latent_kv_prepare": (_i, [_p, _i64, _i, _i, _p, _f, _p, _i, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _p]),
+    "vmx_latent_attention": (_i, [_p, _p, _p, _p, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p]),
+    "vmx_grouped_topk_router": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
+    "vmx_linear_bf16w": (_i, [_p, _i, _p, _i, _p, _i, _i, _i, _i, _p]),
+    "vmx_gesutar_create": (_i, [_p, _p, _p]),
+    "vmx_gesutar_destroy": (None, [_p]),
+    "vmx_gesutar_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
+    "vmx_gesutar_missing_tensors": (_i, [_p]),
+    "vmx_gesutar_forward": (_i, [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _i, _p, _p, _p, _p]),
 }
 
 
@@ -239,6 +248,24 @@ class Gemma4Config(C.Structure):
         ("sliding_window", _i), ("rot_dim_sliding", _i), ("rot_dim_full", _i), ("max_position", _i), ("kv_cache_dtype", _i),
         ("block_size", _i), ("num_blocks", _i), ("max_batch", _i), ("max_seq_len", _i), ("final_logit_softcap", _f),
         ("embed_ggml_type", _i), ("hidden_size_per_layer_input", _i), ("vocab_size_per_layer_input", _i), ("ple_embed_ggml_type", _i), ("tp_size", _i), ("tp_rank", _i), ("max_prefill_tokens", _i),
+    ]
+
+
+class GesutarLayerConfig(C.Structure):
+    """struct vmx_gesutar_layer_config (include/vmx.h)."""
+    _fields_ = [
+        ("mixer", _i), ("heads", _i), ("dim", _i), ("rot_dim", _i), ("vdim", _i), ("kv_rank", _i), ("window", _i), ("rot_dims", _i),
+        ("rot_base", C.c_double), ("scale", _f), ("mlp", _i), ("experts", _i), ("top", _i), ("groups", _i), ("keep_groups", _i),
+        ("expert_ff", _i), ("shared_ff", _i), ("router_scale", _f),
+    ]
+
+
+class GesutarConfig(C.Structure):
+    """struct vmx_gesutar_config (include/vmx.h)."""
+    _fields_ = [
+        ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("embed_scale", C.c_double), ("bigram_buckets", _i),
+        ("bigram_mul_prev", _i), ("bigram_mul_cur", _i), ("dtype", _i), ("block_size", _i), ("num_blocks", _i), ("max_tokens", _i),
+        ("max_seqs", _i),
     ]
 
 

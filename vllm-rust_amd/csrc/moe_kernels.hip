@@ -71,6 +71,102 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void *__restric
     }
 }
 
+// Router with group-limited selection: softmax over all experts; the experts form `groups` equal runs of neighbours, a group's
+// score is its largest probability, and only experts of the `keep` best groups can be chosen; then k rounds of argmax (ties ->
+// smaller index) over what is left.  Weights: the chosen probabilities divided by (their sum + 1e-20), times `scale`.
+// One wave per token; lane l holds experts (and groups) l, l + 64, ...: E <= 256.
+__global__ __launch_bounds__(256) void grouped_topk_router_kernel(const float *__restrict__ logits, float *__restrict__ w_out,
+                                                                   int32_t *__restrict__ id_out, int tokens, int E, int k, int groups,
+                                                                   int keep, float scale) {
+    __shared__ float sc[4][256];
+    __shared__ int32_t ok[4][256];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, t = blockIdx.x * 4 + wave;
+    if (t >= tokens) return;   // no workgroup-wide barrier below: a wave only exchanges with itself
+    float v[4];
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int e = lane + 64 * j;
+        v[j] = e < E ? logits[(int64_t)t * E + e] : -FLT_MAX;
+        mx = fmaxf(mx, v[j]);
+    }
+    mx = vmx_wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        v[j] = (lane + 64 * j < E) ? expf(v[j] - mx) : 0.f;
+        sum += v[j];
+    }
+    sum = vmx_wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = (lane + 64 * j < E) ? v[j] / sum : -FLT_MAX;
+    if (groups > 1 && keep < groups) {
+        const int gs = E / groups;
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc[wave][lane + 64 * j] = v[j];
+        __builtin_amdgcn_wave_barrier();
+        float gv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int g = lane + 64 * j;
+            gv[j] = -FLT_MAX;
+            if (g < groups)
+                for (int i = 0; i < gs; i++) gv[j] = fmaxf(gv[j], sc[wave][g * gs + i]);
+            ok[wave][g] = 0;
+        }
+        __builtin_amdgcn_wave_barrier();
+        for (int r = 0; r < keep; r++) {
+            float bv = -FLT_MAX;
+            int bi = 0x7fffffff;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int g = lane + 64 * j;
+                if (g < groups && gv[j] > bv) { bv = gv[j]; bi = g; }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ov = vmx_lane_xor_m(bv, off);
+                const int oi = vmx_lane_xor_m(bi, off);
+                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (lane + 64 * j == bi) { gv[j] = -FLT_MAX; ok[wave][bi] = 1; }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int e = lane + 64 * j;
+            if (e < E && !ok[wave][e / gs]) v[j] = -FLT_MAX;
+        }
+    }
+    float selected = 0.f;
+    for (int ki = 0; ki < k; ki++) {
+        float bv = -FLT_MAX;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int e = lane + 64 * j;
+            if (e < E && v[j] > bv) { bv = v[j]; bi = e; }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = vmx_lane_xor_m(bv, off);
+            const int oi = vmx_lane_xor_m(bi, off);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) { w_out[(int64_t)t * k + ki] = bv; id_out[(int64_t)t * k + ki] = bi; }
+        selected += bv;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (lane + 64 * j == bi) v[j] = -FLT_MAX;
+    }
+    if (lane == 0) {
+        const float f = scale / (selected + 1e-20f);
+        for (int ki = 0; ki < k; ki++) w_out[(int64_t)t * k + ki] *= f;
+    }
+}
+
 // Single workgroup.  sorted_token_ids: per expert, the flattened (token*k + slot) indices routed to it in
 // ascending order, each expert's run padded to a multiple of block_size with `numel`; expert_ids: the
 // expert of each block; total_tokens_post_pad[0] = padded length.
@@ -275,6 +371,20 @@ extern "C" int vmx_topk_softmax(const void *logits, int logits_dtype, float *top
         hipLaunchKernelGGL(topk_softmax_kernel<false>, grid, block, 0, vmx_stream(stream), logits, topk_weights, topk_ids, tokens, num_experts,
                            k, renormalize, round_probs_bf16);
     VMX_CHECK_LAUNCH("topk_softmax");
+    return VMX_OK;
+}
+
+extern "C" int vmx_grouped_topk_router(const float *logits, float *topk_weights, int32_t *topk_ids, int tokens, int num_experts, int k,
+                                       int groups, int keep_groups, float scale, void *stream) {
+    VMX_REQUIRE(logits && topk_weights && topk_ids, "grouped_topk_router: null pointer");
+    VMX_REQUIRE(num_experts >= 1 && num_experts <= 256, "grouped_topk_router: num_experts (%d) must be in 1..256", num_experts);
+    VMX_REQUIRE(groups >= 1 && num_experts % groups == 0, "grouped_topk_router: %d experts do not form %d equal groups", num_experts, groups);
+    VMX_REQUIRE(keep_groups >= 1 && keep_groups <= groups, "grouped_topk_router: keep_groups (%d) must be in 1..groups", keep_groups);
+    VMX_REQUIRE(k >= 1 && k <= keep_groups * (num_experts / groups), "grouped_topk_router: k (%d) exceeds the experts of the kept groups", k);
+    if (tokens <= 0) return VMX_OK;
+    hipLaunchKernelGGL(grouped_topk_router_kernel, dim3((tokens + 3) / 4), dim3(256), 0, vmx_stream(stream), logits, topk_weights, topk_ids,
+                       tokens, num_experts, k, groups, keep_groups, scale);
+    VMX_CHECK_LAUNCH("grouped_topk_router");
     return VMX_OK;
 }
 

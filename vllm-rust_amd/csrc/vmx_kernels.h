@@ -172,3 +172,30 @@ int vmx_bf16_gemm_nt(uint16_t *y, const uint16_t *x, const uint16_t *w, const ui
 // Q3_K table x 2..16 bf16 rows on the matrix cores (kquant_kernels.hip); f32 out [m][n_out]
 bool vmx_q3k_gemm16_ok(int n_out, int n_in, int m);
 int vmx_q3k_gemm16_bf16(const void *w, const uint16_t *x, float *y, int n_out, int n_in, int m, hipStream_t st);
+
+// linear_generic.hip: linear layers over unquantized bf16 weights of any shape (f32 accumulation in ascending k)
+enum { VMX_EP_STORE = 0, VMX_EP_RELU2 = 1, VMX_EP_ADD_F32 = 2, VMX_EP_MUL_SIGMOID = 3 };
+struct VmxLinear {
+    const void *A = nullptr;           // activations [M, K], K contiguous, rows lda elements apart
+    int a_f32 = 0;                     // 1: f32 activations, 0: bf16
+    int64_t lda = 0;
+    const uint16_t *W = nullptr;       // bf16 weights; element (n, k) at W[n * w_sn + k * w_sk]
+    int64_t w_sn = 0, w_sk = 1;
+    void *C = nullptr;                 // output [M, N], rows ldc elements apart
+    int c_f32 = 0;
+    int64_t ldc = 0;
+    int M = 0, N = 0, K = 0;
+    int batch = 1;                     // independent products on blockIdx.z, operands a_bs / w_bs / c_bs / aux_bs elements apart
+    int64_t a_bs = 0, w_bs = 0, c_bs = 0, aux_bs = 0;
+    const int32_t *row_ids = nullptr;  // output row m reads activation row row_ids[m] / row_div; ids outside [0, row_limit) are padding
+    int row_div = 1, row_limit = 0;
+    const int32_t *block_expert = nullptr;   // row block b (block_rows rows) multiplies with W + block_expert[b] * expert_stride
+    int64_t expert_stride = 0;
+    int block_rows = 0;
+    const int32_t *total_rows = nullptr;     // device scalar: row blocks at or past it do nothing
+    int epilogue = VMX_EP_STORE;       // RELU2: max(v, 0)^2; ADD_F32: C += v (f32 C); MUL_SIGMOID: v * sigmoid(aux[m, n])
+    const float *aux = nullptr;
+    int64_t ldaux = 0;
+    int exact = 0;                     // 1: multiply in f32 on the vector ALU even where the matrix cores could take bf16 operands
+};
+int vmx_linear_launch(const VmxLinear &p, hipStream_t st);
