@@ -19,6 +19,7 @@ int4 GEMV, OpenMP over output columns, on a bounded sample of the same per-token
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -635,6 +636,128 @@ def mixtral_secondary(prompt, steps, warmup, batches=(1, 4, 16)):
             "batch_sweep": by_batch}
 
 
+GESUTAR_SIZES = {
+    # name: (width, layers, heads, dim, rot_dim, vdim, kv_rank, window, experts, top, groups, keep, expert_ff, shared_ff, vocab)
+    "1k": (1024, 4, 8, 64, 32, 64, 256, 1024, 16, 4, 4, 2, 512, 512, 32000),
+    "2k": (2048, 4, 16, 128, 64, 128, 512, 4096, 32, 4, 4, 2, 1024, 1024, 32000),
+}
+
+
+def _timed_graph(fn, side, warmup, steps):
+    """fn captured into one hipGraph on `side`, replayed warmup + steps times; seconds per replay."""
+    with torch.cuda.stream(side):
+        fn()
+        g = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            fn()
+        for _ in range(warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        del g
+    return dt
+
+
+def gesutar_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16)):
+    """Gesutar (latent attention + grouped-router MoE, bf16 weights) at layer sizes of real models, beside the closest existing
+    model at equal size: the unquantized bf16 Qwen3 executor with the same width, depth, head count and per-token feed-forward
+    width (top x expert_ff + shared_ff).  Prompt pass: tokens/s of one `prompt`-token sequence; decode: aggregate tok/s of B
+    sequences at context `prompt`, one hipGraph per step.  Random-init weights."""
+    from vllm_rust_amd.gesutar import GesutarForCausalLM, GesutarLayerSpec, GesutarSpec, synthetic_weights
+    from vllm_rust_amd.qwen3 import QuantizedQwen3ForCausalLM, Qwen3Spec
+    out = {}
+    dev = torch.device("cuda", torch.cuda.current_device())
+    side = torch.cuda.Stream(device=dev)
+    BM = max(batches)
+    per_seq = (prompt + warmup + steps + 8 + 15) // 16 + 1
+    for name in sizes:
+        W, NL, H, dim, rd, vd, R, win, E, top, G, keep, ff, sff, V = GESUTAR_SIZES[name]
+        layer = GesutarLayerSpec(heads=H, dim=dim, rot_dim=rd, vdim=vd, kv_rank=R, window=win, rot_dims=rd, rot_base=1e6, scale=1.0 / math.sqrt(dim + rd),
+                                 experts=E, top=top, groups=G, keep_groups=keep, expert_ff=ff, shared_ff=sff, router_scale=1.0)
+        spec = GesutarSpec(vocab=V, width=W, layers=[layer] * NL, embed_scale=1.0, bigram_buckets=4093, bigram_mul_prev=31, bigram_mul_cur=7)
+        model = GesutarForCausalLM(spec, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        model.load_state(synthetic_weights(spec, 3, device=dev))
+        i32 = lambda a: torch.as_tensor(a, dtype=torch.int32, device=dev).contiguous()
+        bt = torch.arange(per_seq * BM, dtype=torch.int32, device=dev).reshape(BM, per_seq).contiguous()
+        g = torch.Generator(device=dev).manual_seed(1)
+        toks = torch.randint(0, V, (prompt,), dtype=torch.int32, device=dev, generator=g)
+        prev = torch.cat([i32([-1]), toks[:-1]])
+        pos = torch.arange(prompt, dtype=torch.int32, device=dev)
+        last = i32([prompt - 1])
+        res = {}
+        for b in range(BM):          # fill every sequence's cache (the first pass also pays the lazy set-up)
+            slots = (bt[b, (pos // 16).long()] * 16 + pos % 16).to(torch.int32)
+            sid = torch.full((prompt,), b, dtype=torch.int32, device=dev)
+            model.forward(toks, prev, pos, slots, sid, bt, last, want_logits=False, want_greedy=True)
+        torch.cuda.synchronize()
+        slots0 = (bt[0, (pos // 16).long()] * 16 + pos % 16).to(torch.int32)
+        sid0 = torch.zeros(prompt, dtype=torch.int32, device=dev)
+        t = _timed_graph(lambda: model.forward(toks, prev, pos, slots0, sid0, bt, last, want_logits=False, want_greedy=True), side, 2, 10)
+        lin = NL * (W * (H * (dim + rd) + R + rd + H * vd) + H * dim * R + H * vd * R + H * vd * W + (top * 2 * ff + 2 * sff + E) * W)
+        att = NL * H * (2 * R + rd) * min(win, prompt / 2)
+        res["prefill"] = {"tokens": prompt, "ms": round(t * 1e3, 3), "tok_s": round(prompt / t, 1),
+                          "TFLOP_s": round(2.0 * prompt * (lin + att + V * W / prompt) / t / 1e12, 2)}
+        wbytes = 2 * (NL * (W * (H * (dim + rd) + R + rd + H * vd) + H * dim * R + H * vd * R + H * vd * W + (2 * sff + E) * W) + V * W)
+        for B in batches:
+            dtok = torch.randint(0, V, (B,), dtype=torch.int32, device=dev, generator=g)
+            dprev = torch.randint(0, V, (B,), dtype=torch.int32, device=dev, generator=g)
+            dpos = torch.full((B,), prompt, dtype=torch.int32, device=dev)
+            dslots = (bt[:B, prompt // 16] * 16 + prompt % 16).to(torch.int32).contiguous()
+            dsid = torch.arange(B, dtype=torch.int32, device=dev)
+            rows = torch.arange(B, dtype=torch.int32, device=dev)
+            t = _timed_graph(lambda: model.forward(dtok, dprev, dpos, dslots, dsid, bt, rows, want_logits=False, want_greedy=True), side, warmup, steps)
+            experts_hit = min(E, B * top)
+            by = wbytes + 2 * NL * experts_hit * 2 * ff * W + 2 * NL * B * min(win, prompt + 1) * (R + rd)
+            res[f"decode_b{B}"] = {"tok_s": round(B / t, 1), "ms_per_step": round(t * 1e3, 4), "GBps_algorithmic": round(by / t / 1e9, 1)}
+        model.close()
+        del model
+        # the closest existing model at equal size
+        I = top * ff + sff
+        qs = Qwen3Spec(W, NL, H, max(1, H // 4), dim + rd if (dim + rd) in (64, 128) else 128, I, V, max_position=max(4096, prompt + steps + warmup + 16),
+                       num_blocks=per_seq * BM, max_batch=BM, max_seq_len=prompt + steps + warmup + 16, max_prefill_tokens=prompt)
+        qm = QuantizedQwen3ForCausalLM(qs)
+        qm.load_synthetic_bf16(seed=3)
+        ids = torch.empty(BM, dtype=torch.int32, device=dev)
+        btq = bt.flip(0).contiguous()
+        qres = {}
+        with torch.cuda.stream(side):
+            for b in range(BM):
+                qm.prefill(toks, 0, btq[b], out_id=ids[b:b + 1])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                qm.prefill(toks, 0, btq[0], out_id=ids[0:1])
+            torch.cuda.synchronize()
+            t = (time.perf_counter() - t0) / 3
+        nq, nkv = qs.num_heads * qs.head_dim, qs.num_kv_heads * qs.head_dim
+        qlin = NL * (W * (nq + 2 * nkv) + nq * W + 3 * W * I)
+        qres["prefill"] = {"tokens": prompt, "ms": round(t * 1e3, 3), "tok_s": round(prompt / t, 1),
+                           "TFLOP_s": round(2.0 * prompt * (qlin + NL * 2 * nq * prompt / 2 + V * W / prompt) / t / 1e12, 2)}
+        for B in batches:
+            qpos = torch.full((B,), prompt, dtype=torch.int32, device=dev)
+            qslots = (btq[:B, prompt // 16] * 16 + prompt % 16).to(torch.int32).contiguous()
+            sl = torch.full((B,), prompt + 1, dtype=torch.int32, device=dev)
+            qout = torch.empty(B, dtype=torch.int32, device=dev)
+            qids = ids[:B].contiguous()
+            btb = btq[:B].contiguous()
+            t = _timed_graph(lambda: qm.forward_decode_batch(qids, qpos, qslots, btb, sl, max_seq_len=qs.max_seq_len, out_ids=qout), side, warmup, steps)
+            by = 2 * (qlin + V * W) + 2 * NL * B * 2 * nkv * (prompt + 1)
+            qres[f"decode_b{B}"] = {"tok_s": round(B / t, 1), "ms_per_step": round(t * 1e3, 4), "GBps_algorithmic": round(by / t / 1e9, 1)}
+        qm.close()
+        del qm
+        out[name] = {"gesutar": res, "qwen3_bf16_dense": qres,
+                     "config": {"width": W, "layers": NL, "heads": H, "dim": dim, "rot_dim": rd, "vdim": vd, "kv_rank": R, "window": win, "experts": E,
+                                "top": top, "groups": [G, keep], "expert_ff": ff, "shared_ff": sff, "vocab": V,
+                                "qwen3": {"kv_heads": qs.num_kv_heads, "head_dim": qs.head_dim, "intermediate": I}}}
+    return {"metric": "Gesutar prompt and decode throughput beside the bf16 dense Qwen3 executor at equal size", "unit": "tok/s", "dtype": "bf16",
+            "data": "synthetic", "prompt": prompt, "sizes": out}
+
+
 def plan_job(gpus, world, replicas_flag, weights, local_ranks):
     """What a launch of this script measures -- pure argument logic, no device.  N = 1: the single-GPU job.  N > 1 (one process
     per GPU under torch.distributed.run): ONE model tensor-parallel over the N ranks (BASELINE.json's metric is the TP curve at
@@ -791,7 +914,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary measurements (other models at N = 1, replicas at N > 1)")
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
-    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3"], default="all",
+    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
                          "their own block), so that a kernel trace of the run holds that workload's launches only")
     ap.add_argument("--tp", action="store_true", help="accepted for compatibility: with --gpus N > 1 the tensor-parallel job is the default")
@@ -808,8 +931,10 @@ def main():
     plan = plan_job(args.gpus, world, args.replicas, args.weights, d.local)
 
     K_steps, W_steps = args.steps, args.warmup
-    if args.workload in ("gemma4", "mixtral", "exl3"):   # one secondary alone (single GPU)
-        if args.workload == "gemma4":
+    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar"):   # one secondary alone (single GPU)
+        if args.workload == "gesutar":
+            blk = gesutar_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
+        elif args.workload == "gemma4":
             blk = gemma4_secondary(args.prompt, max(16, K_steps // 2), W_steps, cpu_leg=not args.no_cpu_baseline)
         elif args.workload == "mixtral":
             blk = mixtral_secondary(args.prompt, max(16, K_steps // 2), W_steps)

@@ -311,7 +311,7 @@ extern "C" void vmx_gesutar_destroy(vmx_gesutar *m) {
 
 // One checkpoint tensor by its name in the file (bf16, shape [out, in] for matrices).  `data` may be host or device memory.
 extern "C" int vmx_gesutar_load_tensor(vmx_gesutar *m, const char *name, const void *data, size_t bytes, void *stream) {
-    VMX_REQUIRE(m && name && data, "gesutar_load_tensor: null pointer");
+    VMX_REQUIRE(m && name && (data || bytes == 0), "gesutar_load_tensor: null pointer");
     hipStream_t st = vmx_stream(stream);
     const vmx_gesutar_config &c = m->cfg;
     const size_t W = c.width;
@@ -361,7 +361,8 @@ extern "C" int vmx_gesutar_load_tensor(vmx_gesutar *m, const char *name, const v
     }
     VMX_REQUIRE(dst, "gesutar_load_tensor: unknown tensor `%s`", name);
     VMX_REQUIRE(bytes == need, "gesutar_load_tensor: `%s`: expected %zu bytes of bf16, got %zu", name, need, bytes);
-    if (int rc = upload(*dst, off, data, bytes, st)) return rc;
+    if (bytes > 0)
+        if (int rc = upload(*dst, off, data, bytes, st)) return rc;
     erase_name(*missing, n);
     return VMX_OK;
 }

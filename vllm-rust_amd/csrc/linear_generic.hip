@@ -97,6 +97,133 @@ __global__ __launch_bounds__(256) void linear_fma_kernel(const VmxLinear p) {
     }
 }
 
+// Matrix-core form: BM x 64 output tile, 64-deep k stages of bf16 in LDS (rows padded by 16 bytes), v_mfma_f32_16x16x32_bf16.
+// BM = 64: wave w owns the 32 x 32 quadrant (w >> 1, w & 1) as 2 x 2 instruction tiles; BM = 16: wave w owns columns 16 w .. + 16.
+// The next stage is requested into registers before the current one is multiplied.  An output element sums its k in the same
+// order in both shapes, so a row's result does not depend on which shape its call took.
+template <int BM>
+__global__ __launch_bounds__(256) void linear_mfma_kernel(const VmxLinear p) {
+    constexpr int BN = 64, BK = 64, LD = BK + 8, CH = BK / 8;   // CH: 8-element chunks per staged row
+    constexpr int TI = BM == 64 ? 2 : 1, TJ = BM == 64 ? 2 : 1;
+    constexpr int ACH = (BM * CH + 255) / 256, WCH = BN * CH / 256;
+    __shared__ __align__(16) uint16_t As[BM * LD];
+    __shared__ __align__(16) uint16_t Ws[BN * LD];
+    __shared__ int64_t rows[BM];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN, z = blockIdx.z;
+    if (p.total_rows && m0 >= *p.total_rows) return;
+    const uint16_t *W = p.W + z * p.w_bs;
+    if (p.block_expert) W += (int64_t)p.block_expert[m0 / p.block_rows] * p.expert_stride;
+    const int64_t a_off = z * p.a_bs;
+    for (int i = tid; i < BM; i += 256) rows[i] = linear_src_row(p, m0 + i);
+    __syncthreads();
+    // 16-byte loads need aligned rows: every row start and every chunk a multiple of 8 (bf16) elements
+    const bool a_vec = (p.K & 7) == 0 && (p.lda & 7) == 0 && (a_off & 7) == 0 && ((uintptr_t)p.A & 31) == 0;
+    const bool w_vec = p.w_sk == 1 && (p.K & 7) == 0 && (p.w_sn & 7) == 0 && (((uintptr_t)W) & 15) == 0;
+    uint4 ar[ACH], wr[WCH];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < ACH; c++) {
+            const int idx = tid + 256 * c, m = idx / CH, k = k0 + 8 * (idx % CH);
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (idx < BM * CH) {
+                const int64_t r = rows[m];
+                if (r >= 0 && k < p.K) {
+                    const int64_t at = a_off + r * p.lda + k;
+                    if (a_vec) {
+                        if (p.a_f32) {
+                            const float4 f0 = *reinterpret_cast<const float4 *>((const float *)p.A + at);
+                            const float4 f1 = *reinterpret_cast<const float4 *>((const float *)p.A + at + 4);
+                            const float f[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
+                            v = vmx_pack16x8<false>(f);
+                        } else {
+                            v = *reinterpret_cast<const uint4 *>((const uint16_t *)p.A + at);
+                        }
+                    } else {
+                        float f[8];
+#pragma unroll
+                        for (int e = 0; e < 8; e++) f[e] = k + e < p.K ? ld_act(p.A, p.a_f32, at + e) : 0.f;
+                        v = vmx_pack16x8<false>(f);
+                    }
+                }
+            }
+            ar[c] = v;
+        }
+#pragma unroll
+        for (int c = 0; c < WCH; c++) {
+            const int idx = tid + 256 * c, n = n0 + idx / CH, k = k0 + 8 * (idx % CH);
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (n < p.N && k < p.K) {
+                if (w_vec) {
+                    v = *reinterpret_cast<const uint4 *>(W + (int64_t)n * p.w_sn + k);
+                } else {
+                    uint32_t h[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) h[e] = k + e < p.K ? W[(int64_t)n * p.w_sn + (int64_t)(k + e) * p.w_sk] : 0;
+                    v = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+                }
+            }
+            wr[c] = v;
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int c = 0; c < ACH; c++) {
+            const int idx = tid + 256 * c;
+            if (idx < BM * CH) *reinterpret_cast<uint4 *>(As + (idx / CH) * LD + 8 * (idx % CH)) = ar[c];
+        }
+#pragma unroll
+        for (int c = 0; c < WCH; c++) {
+            const int idx = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(Ws + (idx / CH) * LD + 8 * (idx % CH)) = wr[c];
+        }
+    };
+    vmx_f32x4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++) acc[i][j] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int wm = BM == 64 ? (wave >> 1) * 32 : 0, wn = BM == 64 ? (wave & 1) * 32 : wave * 16;
+    const int fl = lane & 15, fg = lane >> 4;
+    fetch(0);
+    stash();
+    __syncthreads();
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+        if (k0 + BK < p.K) fetch(k0 + BK);
+#pragma unroll
+        for (int s = 0; s < BK / 32; s++) {
+            uint4 af[TI], wf[TJ];
+#pragma unroll
+            for (int i = 0; i < TI; i++) af[i] = *reinterpret_cast<const uint4 *>(As + (wm + 16 * i + fl) * LD + 32 * s + 8 * fg);
+#pragma unroll
+            for (int j = 0; j < TJ; j++) wf[j] = *reinterpret_cast<const uint4 *>(Ws + (wn + 16 * j + fl) * LD + 32 * s + 8 * fg);
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, af[i]), __builtin_bit_cast(vmx_bf16x8, wf[j]),
+                                                                        acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+        if (k0 + BK < p.K) {
+            stash();
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int ml = wm + 16 * i + 4 * fg + r, m = m0 + ml;
+            if (m >= p.M || (p.row_ids && rows[ml] < 0)) continue;
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const int n = n0 + wn + 16 * j + fl;
+                if (n < p.N) linear_store(p, z, m, n, acc[i][j][r]);
+            }
+        }
+}
+
 }  // namespace
 
 int vmx_linear_launch(const VmxLinear &p, hipStream_t st) {
@@ -109,8 +236,13 @@ int vmx_linear_launch(const VmxLinear &p, hipStream_t st) {
     if (p.M == 0) return VMX_OK;
     const int bm = p.block_expert ? p.block_rows : (p.M <= 16 ? 16 : 64);
     dim3 grid((p.N + 63) / 64, (p.M + bm - 1) / bm, p.batch);
-    if (bm == 16) hipLaunchKernelGGL(linear_fma_kernel<16>, grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(linear_fma_kernel<64>, grid, dim3(256), 0, st, p);
+    if (p.exact) {
+        if (bm == 16) hipLaunchKernelGGL(linear_fma_kernel<16>, grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(linear_fma_kernel<64>, grid, dim3(256), 0, st, p);
+    } else {
+        if (bm == 16) hipLaunchKernelGGL(linear_mfma_kernel<16>, grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(linear_mfma_kernel<64>, grid, dim3(256), 0, st, p);
+    }
     VMX_CHECK_LAUNCH("linear");
     return VMX_OK;
 }

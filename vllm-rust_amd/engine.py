@@ -20,7 +20,8 @@ from ._lib import check, lib
 
 
 class BlockManager:
-    """Free list of cache blocks.  Freed blocks are handed out again first (LIFO), so reuse is the common case, not the corner."""
+    """Free list of cache blocks.  Freed blocks are handed out again first, last freed first, so reuse (in another order than
+    the first owner's) is the common case, not the corner."""
 
     def __init__(self, num_blocks: int, block_size: int):
         self.num_blocks, self.block_size = num_blocks, block_size
@@ -38,7 +39,7 @@ class BlockManager:
         return [self.free.pop() for _ in range(n)]
 
     def release(self, blocks: list) -> None:
-        self.free.extend(reversed(blocks))
+        self.free.extend(blocks)
 
 
 @dataclasses.dataclass

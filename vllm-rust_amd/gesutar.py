@@ -139,20 +139,26 @@ class GesutarSpec:
         return out
 
 
-def synthetic_weights(spec: GesutarSpec, seed: int = 0) -> dict:
-    """Seeded random-init checkpoint of the architecture (bf16 host tensors): matrices ~ 1 / sqrt(in), norm weights around 1,
-    sinks around 0, so that activations stay O(1) through the stack."""
-    g = torch.Generator().manual_seed(seed)
+def synthetic_weights(spec: GesutarSpec, seed: int = 0, device="cpu") -> dict:
+    """Seeded random-init checkpoint of the architecture (bf16 tensors on `device`): matrices ~ 1 / sqrt(in), norm weights
+    around 1, sinks around 0, so that activations stay O(1) through the stack."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    _randn = torch.randn
+
+    class torch_:   # every draw on the generator's device
+        @staticmethod
+        def randn(shape, generator):
+            return _randn(shape, generator=generator, device=device)
     ck = {}
     for name, shape in spec.tensor_shapes().items():
         if name.endswith("norm1") or name.endswith("norm2") or name.endswith(".norm"):
-            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            t = 1.0 + 0.1 * torch_.randn(shape, generator=g)
         elif name.endswith("sink"):
-            t = 0.5 * torch.randn(shape, generator=g)
+            t = 0.5 * torch_.randn(shape, generator=g)
         elif name in ("embed", "bigram"):
-            t = torch.randn(shape, generator=g) * (0.5 if name == "bigram" else 1.0 / max(spec.embed_scale, 1e-6))
+            t = torch_.randn(shape, generator=g) * (0.5 if name == "bigram" else 1.0 / max(spec.embed_scale, 1e-6))
         else:
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+            t = torch_.randn(shape, generator=g) / math.sqrt(shape[-1])
         ck[name] = t.to(torch.bfloat16)
     return ck
 
@@ -242,11 +248,11 @@ class GesutarForCausalLM:
         Returns (logits f32 [n, vocab] or None, greedy ids int32 [n] or None, trace f32 [layers, T, width] or None)."""
         T = tokens.numel()
         n = 0 if logit_rows is None else logit_rows.numel()
-        logits = torch.empty((n, self.spec.vocab), dtype=torch.float32, device=self.device) if (n and want_logits) else None
+        logits = torch.empty((n, self.spec.vocab), dtype=torch.float32, device=self.device) if n else None
         ids = torch.empty(n, dtype=torch.int32, device=self.device) if (n and want_greedy) else None
         trace = torch.empty((len(self.spec.layers), T, self.spec.width), dtype=torch.float32, device=self.device) if layer_trace else None
         check(lib.vmx_gesutar_forward(self._h, tokens.data_ptr(), prev_tokens.data_ptr(), positions.data_ptr(), slots.data_ptr(),
                                       seq_ids.data_ptr(), T, block_tables.data_ptr(), block_tables.shape[0], block_tables.shape[1],
                                       None if not n else logit_rows.data_ptr(), n, None if logits is None else logits.data_ptr(),
                                       None if ids is None else ids.data_ptr(), None if trace is None else trace.data_ptr(), self._stream()))
-        return logits, ids, trace
+        return (logits if want_logits else None), ids, trace
