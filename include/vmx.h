@@ -955,11 +955,15 @@ int vmx_latent_kv_prepare(const float *fused, int64_t ld_fused, int q_offset, in
  * (window 0: every earlier key), p = softmax((q_abs[t, h] . c_j + q_rot[t, h] . k_rot_j) * scale) whose denominator also holds
  * exp(sink_bf16[h]) when sink_bf16 is given (a key-less, unscaled term).  q_abs is the query mapped into the latent space
  * (U_h^T q_h); the caller maps out_latent through the value up-projection.  Cache rows are found through block_tables
- * [sequences, max_blocks_per_seq] (row = block * block_size + position % block_size).  All f32 except the cache (VMX_F32 / VMX_BF16). */
+ * [sequences, max_blocks_per_seq] (row = block * block_size + position % block_size).  All f32 except the cache (VMX_F32 / VMX_BF16).
+ * Over a bf16 cache with kv_rank and rot_dim multiples of 8 the products run on the matrix cores (queries and softmax weights
+ * enter as bf16 and as a bf16 pair); launches with few rows split the keys over partitions kept in `workspace`
+ * (vmx_latent_attention_workspace_bytes; NULL / too small: no split). */
+size_t vmx_latent_attention_workspace_bytes(int tokens, int heads, int kv_rank, int window, int max_blocks_per_seq, int block_size);
 int vmx_latent_attention(float *out_latent, const float *q_abs, const float *q_rot, const void *cache, int cache_dtype,
                          const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
                          const uint16_t *sink_bf16, float scale, int window, int tokens, int heads, int kv_rank, int rot_dim,
-                         int block_size, void *stream);
+                         int block_size, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Router with group-limited selection: softmax over all experts (f32 logits [tokens, num_experts <= 256]); the experts form
  * `groups` equal runs of neighbours, a group's score is its largest probability, only experts of the keep_groups best groups can

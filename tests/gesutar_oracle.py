@@ -96,6 +96,23 @@ def grouped_router(z, experts, groups, keep, top, scale):
     return ids, torch.stack(wts)
 
 
+def router_margin(z, experts, groups, keep, top):
+    """Smallest relative gap, over the rows of z, between what the router keeps and what it drops (last kept group against first
+    dropped group, last chosen expert against first dropped candidate).  A test in reduced precision is only meaningful on
+    inputs whose margin is well above that precision's rounding."""
+    p = torch.softmax(z.to(F), -1)
+    size, worst = experts // groups, 1.0
+    for row in p:
+        gs = sorted((float(row[g * size:(g + 1) * size].max()) for g in range(groups)), reverse=True)
+        if keep < groups:
+            worst = min(worst, (gs[keep - 1] - gs[keep]) / gs[keep - 1])
+        best = sorted(range(groups), key=lambda g: (-float(row[g * size:(g + 1) * size].max()), g))[:keep]
+        cand = sorted((float(row[e]) for g in best for e in range(g * size, (g + 1) * size)), reverse=True)
+        if top < len(cand):
+            worst = min(worst, (cand[top - 1] - cand[top]) / cand[top - 1])
+    return worst
+
+
 def squared_relu_ff(h, up, down):
     return (torch.relu(h @ up.T) ** 2) @ down.T
 
@@ -111,8 +128,9 @@ def moe(h, w, pre, l):
     return y
 
 
-def forward(spec, weights, tokens, return_layers=False):
-    """Logits [T, vocab] of one sequence from its first token (float64), and the residual stream after every layer."""
+def forward(spec, weights, tokens, return_layers=False, margins=None):
+    """Logits [T, vocab] of one sequence from its first token (float64), and the residual stream after every layer.
+    margins: a list that receives every layer's router_margin."""
     w = {k: v.to(F) for k, v in weights.items()}
     x = embed(tokens, w, spec)
     positions = torch.arange(len(tokens))
@@ -120,7 +138,10 @@ def forward(spec, weights, tokens, return_layers=False):
     for i, l in enumerate(spec.layers):
         x = x + latent_attention(rms_norm(x, w[f"l{i}.norm1"], spec.norm_eps), positions, w, f"l{i}.mix.", l, spec.norm_eps)
         if l.mlp:
-            x = x + moe(rms_norm(x, w[f"l{i}.norm2"], spec.norm_eps), w, f"l{i}.mlp.", l)
+            h2 = rms_norm(x, w[f"l{i}.norm2"], spec.norm_eps)
+            if margins is not None:
+                margins.append(router_margin(h2 @ w[f"l{i}.mlp.router"].T, l.experts, l.groups, l.keep_groups, l.top))
+            x = x + moe(h2, w, f"l{i}.mlp.", l)
         layers.append(x.clone())
     logits = rms_norm(x, w["final.norm"], spec.norm_eps) @ w["head"].T
     return (logits, layers) if return_layers else logits

@@ -54,8 +54,19 @@ def rel_err(got, want):
 TOL = {"float32": 2e-4, "bfloat16": 4e-2}
 
 
-def tokens_for(spec, n, seed):
-    return np.random.default_rng(seed).integers(0, spec.vocab, n).tolist()
+def tokens_for(spec, n, seed, weights=None, extra=0):
+    """n random token ids (+ `extra` more).  With the model's weights: the first draw on which no router decision of the oracle is
+    a close call (relative gap above 1 %), since a decision that bf16 rounding can flip says nothing about the kernels."""
+    from tests import gesutar_oracle as orc
+    for attempt in range(300):
+        toks = np.random.default_rng(seed + 1000 * attempt).integers(0, spec.vocab, n + extra).tolist()
+        if weights is None:
+            return toks
+        margins = []
+        orc.forward(spec, weights, toks, margins=margins)
+        if not margins or min(margins) > 0.01:
+            return toks
+    raise AssertionError("no token draw with safe router margins")
 
 
 # ----------------------------------------------------------------------------- mechanisms alone
@@ -85,10 +96,11 @@ def test_linear_any_shape(gpu, M, N, K, exact):
     g = torch.Generator().manual_seed(M + N + K)
     x = torch.randn((M, K), generator=g)
     w = (torch.randn((N, K), generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    wc = w.cuda()
     for xdt in (torch.float32, torch.bfloat16):
         xc = x.to(xdt).cuda()
         y = torch.empty((M, N), dtype=torch.float32, device="cuda")
-        check(lib.vmx_linear_bf16w(y.data_ptr(), 0, xc.data_ptr(), 0 if xdt == torch.float32 else 1, w.cuda().data_ptr(), M, N, K, exact, None))
+        check(lib.vmx_linear_bf16w(y.data_ptr(), 0, xc.data_ptr(), 0 if xdt == torch.float32 else 1, wc.data_ptr(), M, N, K, exact, None))
         torch.cuda.synchronize()
         xin = xc.cpu().double() if exact else xc.cpu().to(torch.bfloat16).double()
         want = xin @ w.double().T
@@ -111,7 +123,7 @@ def test_linear_rows_do_not_depend_on_the_batch(gpu):
         assert torch.equal(big[77], one[0])
 
 
-def _attention_op(torch, q_abs, q_rot, cache_rows, window, sink, scale, block_size, dtype, shuffle_seed=1):
+def _attention_op(torch, q_abs, q_rot, cache_rows, window, sink, scale, block_size, dtype, shuffle_seed=1, workspace=True):
     """Run vmx_latent_attention for ONE sequence whose key j has the cache row cache_rows[j]; every position is a query.
     The sequence's blocks are scattered over a larger cache."""
     from vllm_rust_amd._lib import check, lib
@@ -130,9 +142,12 @@ def _attention_op(torch, q_abs, q_rot, cache_rows, window, sink, scale, block_si
     pos = torch.arange(T, dtype=torch.int32, device="cuda")
     sk = None if sink is None else sink.to(torch.bfloat16).cuda()
     q_rot_dev = q_rot.float().cuda() if rd else torch.zeros(1, device="cuda")
-    check(lib.vmx_latent_attention(out.data_ptr(), q_abs.float().cuda().data_ptr(), q_rot_dev.data_ptr(), cache.data_ptr(), cdt,
+    nbytes = lib.vmx_latent_attention_workspace_bytes(T, H, R, window, nb, block_size) if workspace else 0
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device="cuda")
+    q_abs_dev = q_abs.float().cuda()                  # every device operand stays referenced until the kernel has run
+    check(lib.vmx_latent_attention(out.data_ptr(), q_abs_dev.data_ptr(), q_rot_dev.data_ptr(), cache.data_ptr(), cdt,
                                    bt.data_ptr(), nb, sid.data_ptr(), pos.data_ptr(), None if sk is None else sk.data_ptr(), scale, window, T, H, R,
-                                   rd, block_size, None))
+                                   rd, block_size, ws.data_ptr() if nbytes else None, nbytes, None))
     torch.cuda.synchronize()
     return out.cpu().double()
 
@@ -150,7 +165,8 @@ def _attention_ref(torch, q_abs, q_rot, rows, window, sink, scale):
     return out
 
 
-@pytest.mark.parametrize("window,use_sink,R,rd,bs", [(9, True, 24, 6, 4), (0, False, 70, 0, 16), (300, True, 130, 16, 8), (1, True, 8, 2, 3)])
+@pytest.mark.parametrize("window,use_sink,R,rd,bs", [(9, True, 24, 6, 4), (0, False, 70, 0, 16), (300, True, 130, 16, 8), (1, True, 8, 2, 3),
+                                                     (70, True, 96, 32, 16), (0, True, 40, 8, 4), (129, False, 512, 64, 16), (64, True, 136, 0, 8)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_latent_attention_op(gpu, window, use_sink, R, rd, bs, dtype):
     vmx, torch = gpu
@@ -161,9 +177,44 @@ def test_latent_attention_op(gpu, window, use_sink, R, rd, bs, dtype):
         rows = rows.to(torch.bfloat16).float()
     q_abs, q_rot = torch.randn((T, H, R), generator=g), torch.randn((T, H, rd), generator=g)
     sink = torch.randn(H, generator=g).to(torch.bfloat16).float() if use_sink else None
-    got = _attention_op(torch, q_abs, q_rot, rows, window, sink, 0.3, bs, dtype)
-    want = _attention_ref(torch, q_abs, q_rot, rows, window, sink, 0.3)
-    assert float((got - want).abs().max()) <= 2e-5
+    # the matrix-core form (bf16 cache, sizes in multiples of 8) takes the queries as bf16
+    mfma = dtype == "bfloat16" and R % 8 == 0 and rd % 8 == 0
+    if mfma:
+        q_abs, q_rot = q_abs.to(torch.bfloat16).float(), q_rot.to(torch.bfloat16).float()
+    want = _attention_ref(torch, q_abs, q_rot, rows, window, sink, 0.3 / math.sqrt(R / 24))
+    for ws in (True, False):                          # with key partitions, and as one walk over all keys
+        got = _attention_op(torch, q_abs, q_rot, rows, window, sink, 0.3 / math.sqrt(R / 24), bs, dtype, workspace=ws)
+        assert float((got - want).abs().max()) <= (1e-4 if mfma else 2e-5)
+
+
+@pytest.mark.parametrize("H", [1, 3, 8, 16, 20])
+def test_latent_attention_mixed_sequences_in_one_tile(gpu, H):
+    """Packed decode tokens of several sequences with different lengths: with fewer than 16 heads one 16-row tile of the
+    matrix-core form holds tokens of different sequences; with more than 16 a token spans two tiles."""
+    from vllm_rust_amd._lib import check, lib
+    vmx, torch = gpu
+    g = torch.Generator().manual_seed(H)
+    R, rd, bs, window = 32, 8, 4, 21
+    lens = [5, 70, 1, 33, 22, 64, 65]
+    S, maxb = len(lens), 20
+    cache = torch.randn((S * maxb * bs, R + rd), generator=g).to(torch.bfloat16)
+    bt = torch.randperm(S * maxb, generator=g).to(torch.int32).reshape(S, maxb)
+    q_abs = torch.randn((S, H, R), generator=g).to(torch.bfloat16).float()
+    q_rot = torch.randn((S, H, rd), generator=g).to(torch.bfloat16).float()
+    sink = torch.randn(H, generator=g).to(torch.bfloat16)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    out = torch.empty((S, H, R), dtype=torch.float32, device="cuda")
+    nbytes = lib.vmx_latent_attention_workspace_bytes(S, H, R, window, maxb, bs)
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device="cuda")
+    dev = [t.cuda() for t in (q_abs, q_rot, cache, bt, torch.arange(S, dtype=torch.int32), pos, sink)]      # kept alive over the launch
+    check(lib.vmx_latent_attention(out.data_ptr(), dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(), 1, dev[3].data_ptr(), maxb,
+                                   dev[4].data_ptr(), dev[5].data_ptr(), dev[6].data_ptr(), 0.25, window, S, H, R, rd, bs,
+                                   ws.data_ptr() if nbytes else None, nbytes, None))
+    torch.cuda.synchronize()
+    for s, n in enumerate(lens):
+        rows = torch.stack([cache[int(bt[s, j // bs]) * bs + j % bs] for j in range(n)]).float()
+        want = _attention_ref(torch, q_abs[s:s + 1].expand(n, H, R), q_rot[s:s + 1].expand(n, H, rd), rows, window, sink.float(), 0.25)[n - 1]
+        assert float((out[s].cpu().double() - want).abs().max()) <= 1e-4, f"sequence {s}"
 
 
 @pytest.mark.parametrize("window", [7, 64, 256, 257])
@@ -210,7 +261,7 @@ def test_whole_prompt_and_layers(gpu, dtype):
     vmx, torch = gpu
     spec = small_spec()
     model, eng, w = build(spec, dtype)
-    toks = tokens_for(spec, 45, 1)
+    toks = tokens_for(spec, 45, 1, w)
     logits, _, trace = eng.step([("a", toks, list(range(45)))], layer_trace=True)
     want, layers = orc.forward(spec, w, toks, return_layers=True)
     for i, l in enumerate(layers):
@@ -246,7 +297,7 @@ def test_cuttings_agree(gpu, dtype):
     spec = small_spec()
     model, eng, w = build(spec, dtype)
     n = 41
-    toks = tokens_for(spec, n, 2)
+    toks = tokens_for(spec, n, 2, w)
     want = orc.forward(spec, w, toks).numpy()
     whole, _, _ = eng.step([("w", toks, list(range(n)))])
     whole = whole.cpu().numpy()
@@ -273,9 +324,9 @@ def test_unequal_batch_against_each_alone(gpu, dtype):
     spec = small_spec()
     model, eng, w = build(spec, dtype)
     lens = [1, 30, 7, 19]
-    prompts = [tokens_for(spec, n, 10 + i) for i, n in enumerate(lens)]
-    tails = [tokens_for(spec, 6, 20 + i) for i in range(4)]
-    want = [orc.forward(spec, w, p + t).numpy() for p, t in zip(prompts, tails)]
+    full = [tokens_for(spec, n, 10 + i, w, extra=6) for i, n in enumerate(lens)]
+    prompts, tails = [f[:n] for f, n in zip(full, lens)], [f[n:] for f, n in zip(full, lens)]
+    want = [orc.forward(spec, w, f).numpy() for f in full]
     lg, _, _ = eng.step([(i, p, list(range(len(p)))) for i, p in enumerate(prompts)])
     lg = lg.cpu().numpy()
     at = 0
@@ -301,7 +352,7 @@ def test_blocks_freed_and_used_again(gpu):
     vmx, torch = gpu
     spec = small_spec()
     model, eng, w = build(spec, "float32", num_blocks=24)
-    a, b = tokens_for(spec, 37, 3), tokens_for(spec, 29, 4)
+    a, b = tokens_for(spec, 37, 3, w), tokens_for(spec, 29, 4, w)
     eng.step([("a", a, [])])
     used = list(eng.seqs["a"].blocks)
     eng.finish("a")
@@ -337,7 +388,7 @@ def test_sharp_attention_at_window_edges(gpu, dtype):
             ck[f"l{i}.mix.sink"].fill_(-4.0)
     model, eng, w = build(spec, dtype, tweak=sharpen)
     n, dec = 30, 40                                   # decoding runs over three windows of the wider layer
-    toks = tokens_for(spec, n + dec, 6)
+    toks = tokens_for(spec, n + dec, 6, w)
     want = orc.forward(spec, w, toks).numpy()
     lg, _, _ = eng.step([("s", toks[:n], list(range(n)))])
     rows = [lg.cpu().numpy()]
@@ -363,7 +414,7 @@ def test_other_sizes(gpu, layer, kw):
     spec = small_spec(layer=layer, **kw)
     for dtype in ("float32", "bfloat16"):
         model, eng, w = build(spec, dtype, seed=3)
-        toks = tokens_for(spec, 23, 7)
+        toks = tokens_for(spec, 23, 7, w)
         want = orc.forward(spec, w, toks).numpy()
         lg, _, _ = eng.step([("a", toks[:17], list(range(17)))])
         rows = [lg.cpu().numpy()]
@@ -441,7 +492,8 @@ def test_trace_replay_tool(gpu, tmp_path):
     (tmp_path / "m").mkdir()
     (tmp_path / "m" / "config.json").write_text(json.dumps(spec.to_config()))
     save_file(ck, str(tmp_path / "m" / "model.safetensors"))
-    a, b = tokens_for(spec, 9, 50), tokens_for(spec, 4, 51)
+    w = {k: v.double() for k, v in ck.items()}
+    a, b = tokens_for(spec, 9, 50, w), tokens_for(spec, 4, 51, w)
     steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:7], "want": [0, 6]}, {"id": "b", "tokens": b, "want": [3]}], "end": ["b"]},
              {"step": 1, "entries": [{"id": "a", "tokens": a[7:8], "want": []}], "end": []},
              {"step": 2, "entries": [{"id": "a", "tokens": a[8:9], "want": [0]}], "end": ["a"]}]
@@ -452,7 +504,6 @@ def test_trace_replay_tool(gpu, tmp_path):
                             "--max-tokens", "64"], input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
         assert r.returncode == 0, r.stderr[-2000:]
         assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
-        w = {k: v.double() for k, v in ck.items()}
         wa, wb = orc.forward(spec, w, a).numpy(), orc.forward(spec, w, b).numpy()
         s0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(3, spec.vocab)
         s2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(1, spec.vocab)

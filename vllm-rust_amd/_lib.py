@@ -212,7 +212,8 @@ _SIGS = {
     "vmx_gemma4_kv_scales_get": (_i, [_p, _i, _p, _p, _p, _p]),
     "vmx_gemma4_debug_kv": (_i, [_p, _i, _i, _i, _p, _sz, _p]),
     "vmx_latent_kv_prepare": (_i, [_p, _i64, _i, _i, _p, _f, _p, _i, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _p]),
-    "vmx_latent_attention": (_i, [_p, _p, _p, _p, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p]),
+    "vmx_latent_attention": (_i, [_p, _p, _p, _p, _i, _p, _i, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p, _sz, _p]),
+    "vmx_latent_attention_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "vmx_grouped_topk_router": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "vmx_linear_bf16w": (_i, [_p, _i, _p, _i, _p, _i, _i, _i, _i, _p]),
     "vmx_gesutar_create": (_i, [_p, _p, _p]),

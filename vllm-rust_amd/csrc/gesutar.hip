@@ -56,7 +56,7 @@ struct vmx_gesutar {
     Buf embed, bigram, final_norm, head;
     std::vector<std::string> missing;
     // step workspaces, sized for max_tokens
-    Buf x, h, fused, qabs, qrot, olat, attn, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
+    Buf x, h, fused, qabs, qrot, olat, attn, attn_ws, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
     int sorted_cap = 0;
     bool f32() const { return cfg.dtype == VMX_F32; }
     size_t esz() const { return f32() ? 4 : 2; }
@@ -179,7 +179,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     m->cfg = c;
     m->layers.resize(c.num_layers);
     const size_t T = c.max_tokens, W = c.width;
-    size_t nf = 0, hr = 0, hrd = 0, hv = 0, ne = 1, pairs = 0, eff = 0, sff = 0, cap = 0;
+    size_t maxr = 0, nf = 0, hr = 0, hrd = 0, hv = 0, ne = 1, pairs = 0, eff = 0, sff = 0, cap = 0;
     int rc = VMX_OK;
 #define GA(buf, n)                       \
     do {                                 \
@@ -258,6 +258,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
             break;
         }
         nf = std::max(nf, (size_t)L.nf);
+        maxr = std::max(maxr, (size_t)lc.kv_rank);
         hr = std::max(hr, (size_t)lc.heads * lc.kv_rank);
         hrd = std::max(hrd, (size_t)lc.heads * lc.rot_dim);
         hv = std::max(hv, ng);
@@ -275,6 +276,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     GA(m->qabs, T * hr * 4);
     GA(m->qrot, T * (hrd + 1) * 4);
     GA(m->olat, T * hr * 4);
+    GA(m->attn_ws, (size_t)24576 * (maxr + 2) * 4);   // key partitions of launches with few rows: tokens x heads x partitions < 24576
     GA(m->attn, T * hv * m->esz());
     GA(m->rlogits, T * ne * 4);
     GA(m->topw, (pairs + 1) * 4);
@@ -303,7 +305,7 @@ extern "C" void vmx_gesutar_destroy(vmx_gesutar *m) {
         for (Buf *b : {&L.norm1, &L.norm2, &L.wfused, &L.dkv_norm, &L.uk, &L.uv, &L.sink, &L.wo, &L.router, &L.eup, &L.edown, &L.sup, &L.sdown,
                        &L.inv_freq, &L.cache})
             b->release();
-    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->rlogits,
+    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->attn_ws, &m->rlogits,
                    &m->topw, &m->topi, &m->sorted, &m->blk_expert, &m->total, &m->inv, &m->act, &m->ydown, &m->sact, &m->sout, &m->hsel})
         b->release();
     delete m;
@@ -430,7 +432,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         }
         if (int rc = vmx_latent_attention(m->olat.as<float>(), m->qabs.as<float>(), m->qrot.as<float>(), L.cache.p, cdt, block_tables,
                                           max_blocks_per_seq, seq_ids, positions, L.sink.as<uint16_t>(), lc.scale, lc.window, T, H, R, rd,
-                                          c.block_size, st))
+                                          c.block_size, m->attn_ws.p, m->attn_ws.bytes, st))
             return rc;
         {   // v_h = V_h o_h, times sigmoid(gate): per head, [T, R] x [vd, R]^T
             VmxLinear v;

@@ -178,6 +178,238 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float *__restrict__ ou
         out[((int64_t)t * H + h) * R + d] = ((part[d] + part[R + d]) + (part[2 * R + d] + part[3 * R + d])) * inv;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// Matrix-core form (bf16 cache).  A workgroup owns a ROW TILE: 16 (token, head) rows = TPT consecutive tokens x HPT heads, which
+// share their keys because the heads of a token read the same cache rows; with 16 or more heads a tile is one token, so decode
+// steps fill the matrix instruction as well as prompts do.  Keys are walked in tiles of 64:
+//   S = Q K^T     wave w takes keys 16 w .. 16 w + 15 of the tile: Q fragments (the latent-space query | rotated part, rounded to
+//                 bf16) stay in registers, key fragments come straight from the cache rows; v_mfma_f32_16x16x32_bf16 leaves lane
+//                 (g, n) the scores of rows 4 g .. 4 g + 3 against key n, so a row's maximum and sum are DPP reductions over 16 lanes
+//                 plus one exchange between the four waves through LDS;
+//   O += P C      the tile's latents are staged TRANSPOSED in LDS ([latent dim][key], lane = key while staging, so the 2-byte
+//                 writes of a wave fall into consecutive banks) and wave w owns a quarter of the latent dimensions; P goes through
+//                 LDS as a bf16 pair hi + lo (two products), which keeps the softmax weights at f32 precision.
+// A tile whose tokens belong to several sequences (decode steps of models with fewer than 16 heads) is processed once per
+// sequence with the other rows masked.  blockIdx.y splits the key range into partitions for launches with few row tiles; their
+// (max, sum, O) triples are merged, with the sink, by latent_attn_merge_kernel.
+struct LatentAttnArgs {
+    float *out;
+    const float *q_abs, *q_rot;
+    const uint16_t *cache;
+    const int32_t *block_tables, *seq_ids, *positions;
+    const uint16_t *sink;
+    float *part_m, *part_l, *part_o;   // [T][H][NP], [T][H][NP], [T][H][NP][R]
+    float scale;
+    int max_blocks, window, T, H, R, rd, block_size, HPT, TPT, NHG, NP;
+};
+
+constexpr int LA_KT = 64, LA_LD = LA_KT + 8;
+
+template <int KSMAX, int DTW>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnArgs a) {
+    extern __shared__ __align__(16) unsigned char la_smem[];
+    const int R = a.R, RW = a.R + a.rd;
+    uint16_t *CT = reinterpret_cast<uint16_t *>(la_smem);            // [R][LA_LD]
+    uint16_t *Phi = CT + (size_t)R * LA_LD;                           // [16][LA_LD]
+    uint16_t *Plo = Phi + 16 * LA_LD;                                 // [16][LA_LD]
+    float *red_max = reinterpret_cast<float *>(Plo + 16 * LA_LD);     // [4][16]
+    float *red_sum = red_max + 64;                                    // [4][16]
+    int32_t *sl = reinterpret_cast<int32_t *>(red_sum + 64);          // [64]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
+    const int tb = blockIdx.x / a.NHG, hg = blockIdx.x % a.NHG, part = blockIdx.y;
+    const int t0 = tb * a.TPT, t_end = min(t0 + a.TPT, a.T);
+    const int ksteps = (RW + 31) >> 5;
+    const int dtiles = (R + 15) >> 4, dt_per_wave = (dtiles + 3) >> 2, dt0 = wave * dt_per_wave;
+    for (int first = t0; first < t_end;) {
+        const int seq = a.seq_ids[first];
+        int last = first;
+        while (last + 1 < t_end && a.seq_ids[last + 1] == seq) last++;
+        const int32_t *bt = a.block_tables + (int64_t)seq * a.max_blocks;
+        const int hi = a.positions[last];
+        const int lo = a.window > 0 ? max(0, a.positions[first] - a.window + 1) : 0;
+        const int ntiles = (hi - lo) / LA_KT + 1, tpp = (ntiles + a.NP - 1) / a.NP;
+        const int kt_begin = part * tpp, kt_end = min(ntiles, kt_begin + tpp);
+        // A operand of S: the query of row fl
+        uint4 qf[KSMAX];
+        {
+            const int tq = t0 + fl / a.HPT, hq = hg * a.HPT + fl % a.HPT;
+            const bool act = fl < a.TPT * a.HPT && tq >= first && tq <= last && hq < a.H;
+#pragma unroll
+            for (int s = 0; s < KSMAX; s++) {
+                const int k = 32 * s + 8 * fg;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (s < ksteps && act && k < RW) {
+                    const float *src = k < R ? a.q_abs + ((int64_t)tq * a.H + hq) * R + k : a.q_rot + ((int64_t)tq * a.H + hq) * a.rd + (k - R);
+                    const float4 f0 = *reinterpret_cast<const float4 *>(src), f1 = *reinterpret_cast<const float4 *>(src + 4);
+                    const float f[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
+                    v = vmx_pack16x8<false>(f);
+                }
+                qf[s] = v;
+            }
+        }
+        // the rows this lane holds in accumulator layout: 4 fg + r
+        int rpos[4], rlo[4], rtok[4], rhead[4];
+        bool ract[4];
+        float m_r[4], l_r[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = 4 * fg + r;
+            rtok[r] = t0 + row / a.HPT;
+            rhead[r] = hg * a.HPT + row % a.HPT;
+            ract[r] = row < a.TPT * a.HPT && rtok[r] >= first && rtok[r] <= last && rhead[r] < a.H;
+            rpos[r] = ract[r] ? a.positions[rtok[r]] : -1;
+            rlo[r] = a.window > 0 ? max(0, rpos[r] - a.window + 1) : 0;
+            m_r[r] = -FLT_MAX;
+            l_r[r] = 0.f;
+        }
+        vmx_f32x4 acc[DTW];
+#pragma unroll
+        for (int d = 0; d < DTW; d++) acc[d] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int kt = kt_begin; kt < kt_end; kt++) {
+            const int kbase = lo + LA_KT * kt;
+            __syncthreads();   // the previous tile's CT / P have been read
+            if (tid < LA_KT) {
+                const int j = kbase + tid;
+                sl[tid] = j <= hi ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+            }
+            __syncthreads();
+            // latents of the tile, transposed: lane = key, wave w takes the 8-wide dimension chunks w, w + 4, ...
+            {
+                const int slot = sl[lane];
+                for (int dc = wave; dc < (R >> 3); dc += 4) {
+                    uint4 v = make_uint4(0, 0, 0, 0);
+                    if (slot >= 0) v = *reinterpret_cast<const uint4 *>(a.cache + (int64_t)slot * RW + 8 * dc);
+                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        CT[(8 * dc + 2 * e) * LA_LD + lane] = (uint16_t)(w4[e] & 0xFFFFu);
+                        CT[(8 * dc + 2 * e + 1) * LA_LD + lane] = (uint16_t)(w4[e] >> 16);
+                    }
+                }
+            }
+            // scores of this wave's 16 keys
+            vmx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+            {
+                const int slot = sl[16 * wave + fl];
+                uint4 kf[KSMAX];
+#pragma unroll
+                for (int s = 0; s < KSMAX; s++) {
+                    const int k = 32 * s + 8 * fg;
+                    kf[s] = make_uint4(0, 0, 0, 0);
+                    if (s < ksteps && slot >= 0 && k < RW) kf[s] = *reinterpret_cast<const uint4 *>(a.cache + (int64_t)slot * RW + k);
+                }
+#pragma unroll
+                for (int s = 0; s < KSMAX; s++)
+                    if (s < ksteps)
+                        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, qf[s]), __builtin_bit_cast(vmx_bf16x8, kf[s]), sacc,
+                                                                       0, 0, 0);
+            }
+            const int j = kbase + 16 * wave + fl;
+            bool ok[4];
+            float sc[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                ok[r] = ract[r] && j <= rpos[r] && j >= rlo[r];
+                sc[r] = ok[r] ? sacc[r] * a.scale : -FLT_MAX;
+                const float mx = vmx_row16_max(sc[r]);
+                if (fl == 0) red_max[wave * 16 + 4 * fg + r] = mx;
+            }
+            __syncthreads();   // maxima and the transposed latents are in LDS
+            float alpha[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int row = 4 * fg + r;
+                const float tm = fmaxf(fmaxf(red_max[row], red_max[16 + row]), fmaxf(red_max[32 + row], red_max[48 + row]));
+                const float m_new = fmaxf(m_r[r], tm);
+                const float p = ok[r] ? expf(sc[r] - m_new) : 0.f;
+                const uint16_t ph = vmx_f32_to_bf16(p);
+                Phi[row * LA_LD + 16 * wave + fl] = ph;
+                Plo[row * LA_LD + 16 * wave + fl] = vmx_f32_to_bf16(p - vmx_bf16_to_f32(ph));
+                const float sm = vmx_row16_sum(p);
+                if (fl == 0) red_sum[wave * 16 + row] = sm;
+                alpha[r] = expf(m_r[r] - m_new);   // both -FLT_MAX (nothing seen yet): 1, and l and acc are still 0
+                m_r[r] = m_new;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int row = 4 * fg + r;
+                l_r[r] = l_r[r] * alpha[r] + ((red_sum[row] + red_sum[16 + row]) + (red_sum[32 + row] + red_sum[48 + row]));
+            }
+#pragma unroll
+            for (int d = 0; d < DTW; d++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[d][r] *= alpha[r];
+#pragma unroll
+            for (int ks = 0; ks < LA_KT / 32; ks++) {
+                const uint4 ah = *reinterpret_cast<const uint4 *>(Phi + fl * LA_LD + 32 * ks + 8 * fg);
+                const uint4 al = *reinterpret_cast<const uint4 *>(Plo + fl * LA_LD + 32 * ks + 8 * fg);
+#pragma unroll
+                for (int d = 0; d < DTW; d++) {
+                    if (d < dt_per_wave && dt0 + d < dtiles) {
+                        const int dim = min(16 * (dt0 + d) + fl, R - 1);
+                        const uint4 cf = *reinterpret_cast<const uint4 *>(CT + dim * LA_LD + 32 * ks + 8 * fg);
+                        acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, ah), __builtin_bit_cast(vmx_bf16x8, cf), acc[d], 0, 0,
+                                                                         0);
+                        acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, al), __builtin_bit_cast(vmx_bf16x8, cf), acc[d], 0, 0,
+                                                                         0);
+                    }
+                }
+            }
+        }
+        // results of rows 4 fg + r, latent dimensions 16 (dt0 + d) + fl
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            if (!ract[r]) continue;
+            const int64_t th = (int64_t)rtok[r] * a.H + rhead[r];
+            if (a.NP == 1) {
+                const float sk = a.sink ? vmx_bf16_to_f32(a.sink[rhead[r]]) : -FLT_MAX;
+                const float M = fmaxf(m_r[r], sk), w = expf(m_r[r] - M);
+                const float den = l_r[r] * w + (a.sink ? expf(sk - M) : 0.f);
+                const float f = den > 0.f ? w / den : 0.f;
+#pragma unroll
+                for (int d = 0; d < DTW; d++) {
+                    const int dim = 16 * (dt0 + d) + fl;
+                    if (d < dt_per_wave && dim < R) a.out[th * R + dim] = acc[d][r] * f;
+                }
+            } else {
+                const int64_t tp = th * a.NP + part;
+                if (wave == 0 && fl == 0) {
+                    a.part_m[tp] = m_r[r];
+                    a.part_l[tp] = l_r[r];
+                }
+#pragma unroll
+                for (int d = 0; d < DTW; d++) {
+                    const int dim = 16 * (dt0 + d) + fl;
+                    if (d < dt_per_wave && dim < R) a.part_o[tp * R + dim] = acc[d][r];
+                }
+            }
+        }
+        first = last + 1;
+    }
+}
+
+// out[t, h] = sum_p e^(m_p - M) O_p / (sum_p e^(m_p - M) l_p + e^(sink - M)), M = max(sink, max_p m_p)
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(float *__restrict__ out, const float *__restrict__ part_m,
+                                                                 const float *__restrict__ part_l, const float *__restrict__ part_o,
+                                                                 const uint16_t *__restrict__ sink, int H, int R, int NP) {
+    const int64_t th = blockIdx.x;
+    const float sk = sink ? vmx_bf16_to_f32(sink[th % H]) : -FLT_MAX;
+    float M = sk;
+    for (int p = 0; p < NP; p++) M = fmaxf(M, part_m[th * NP + p]);
+    float den = sink ? expf(sk - M) : 0.f;
+    for (int p = 0; p < NP; p++) den += expf(part_m[th * NP + p] - M) * part_l[th * NP + p];
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    for (int d = threadIdx.x; d < R; d += 256) {
+        float v = 0.f;
+        for (int p = 0; p < NP; p++) {
+            const float l = part_l[th * NP + p];
+            if (l > 0.f) v = fmaf(expf(part_m[th * NP + p] - M), part_o[(th * NP + p) * R + d], v);
+        }
+        out[th * R + d] = v * inv;
+    }
+}
+
 }  // namespace
 
 extern "C" int vmx_latent_kv_prepare(const float *fused, int64_t ld_fused, int q_offset, int dkv_offset, const uint16_t *latent_norm_w,
@@ -200,22 +432,75 @@ extern "C" int vmx_latent_kv_prepare(const float *fused, int64_t ld_fused, int q
     return VMX_OK;
 }
 
+// Partition count of the matrix-core form for a launch (host arithmetic only): 1 when there are enough row tiles to fill the
+// device, else enough key partitions to give every compute unit a workgroup.
+static int latent_attn_partitions(int tokens, int heads, int window, int max_blocks_per_seq, int block_size) {
+    const int hpt = heads < 16 ? heads : 16, tpt = 16 / hpt, nhg = (heads + hpt - 1) / hpt;
+    const int64_t tiles = (int64_t)((tokens + tpt - 1) / tpt) * nhg;
+    int64_t max_keys = (int64_t)max_blocks_per_seq * block_size;
+    if (window > 0 && window < max_keys) max_keys = window;
+    const int64_t key_tiles = max_keys / LA_KT + 1;
+    if (tiles >= 512) return 1;
+    int64_t np = (1024 + tiles - 1) / tiles;
+    if (np > key_tiles) np = key_tiles;
+    if (np > 64) np = 64;
+    return np < 1 ? 1 : (int)np;
+}
+
+extern "C" size_t vmx_latent_attention_workspace_bytes(int tokens, int heads, int kv_rank, int window, int max_blocks_per_seq,
+                                                       int block_size) {
+    if (tokens <= 0 || heads <= 0 || kv_rank <= 0 || max_blocks_per_seq <= 0 || block_size <= 0) return 0;
+    const int np = latent_attn_partitions(tokens, heads, window, max_blocks_per_seq, block_size);
+    return np == 1 ? 0 : (size_t)tokens * heads * np * (kv_rank + 2) * sizeof(float);
+}
+
 extern "C" int vmx_latent_attention(float *out_latent, const float *q_abs, const float *q_rot, const void *cache, int cache_dtype,
                                     const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
                                     const uint16_t *sink_bf16, float scale, int window, int tokens, int heads, int kv_rank, int rot_dim,
-                                    int block_size, void *stream) {
+                                    int block_size, void *workspace, size_t workspace_bytes, void *stream) {
     VMX_REQUIRE(out_latent && q_abs && q_rot && cache && block_tables && seq_ids && positions, "latent_attention: null pointer");
     VMX_REQUIRE(cache_dtype == VMX_F32 || cache_dtype == VMX_BF16, "latent_attention: the cache holds f32 or bf16");
     VMX_REQUIRE(kv_rank >= 1 && kv_rank <= 512, "latent_attention: kv_rank (%d) must be in 1..512", kv_rank);
     VMX_REQUIRE(heads >= 1 && rot_dim >= 0 && block_size >= 1 && max_blocks_per_seq >= 1 && window >= 0, "latent_attention: bad sizes");
     if (tokens <= 0) return VMX_OK;
+    hipStream_t st = vmx_stream(stream);
+    const int RW = kv_rank + rot_dim;
+    // matrix-core form: bf16 cache, 16-byte chunks of a row must not straddle the latent / rotated boundary
+    if (cache_dtype == VMX_BF16 && kv_rank % 8 == 0 && rot_dim % 8 == 0 && RW <= 576) {
+        LatentAttnArgs a;
+        a.out = out_latent, a.q_abs = q_abs, a.q_rot = q_rot, a.cache = (const uint16_t *)cache;
+        a.block_tables = block_tables, a.seq_ids = seq_ids, a.positions = positions, a.sink = sink_bf16;
+        a.scale = scale, a.max_blocks = max_blocks_per_seq, a.window = window, a.T = tokens, a.H = heads, a.R = kv_rank, a.rd = rot_dim;
+        a.block_size = block_size;
+        a.HPT = heads < 16 ? heads : 16, a.TPT = 16 / a.HPT, a.NHG = (heads + a.HPT - 1) / a.HPT;
+        a.NP = latent_attn_partitions(tokens, heads, window, max_blocks_per_seq, block_size);
+        const size_t need = a.NP == 1 ? 0 : (size_t)tokens * heads * a.NP * (kv_rank + 2) * sizeof(float);
+        if (need > workspace_bytes || (need && !workspace)) a.NP = 1;   // no room for partitions: one workgroup walks all keys
+        a.part_m = (float *)workspace;
+        a.part_l = a.part_m + (size_t)tokens * heads * a.NP;
+        a.part_o = a.part_l + (size_t)tokens * heads * a.NP;
+        const size_t lds = ((size_t)kv_rank * LA_LD + 2 * 16 * LA_LD) * 2 + (64 + 64) * 4 + 64 * 4;
+        dim3 grid((unsigned)(((tokens + a.TPT - 1) / a.TPT) * a.NHG), a.NP);
+        const bool small = RW <= 160 && kv_rank <= 128;
+        const void *fn = small ? (const void *)latent_attn_mfma_kernel<5, 2> : (const void *)latent_attn_mfma_kernel<18, 8>;
+        if (lds > 64 * 1024) VMX_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (small) hipLaunchKernelGGL((latent_attn_mfma_kernel<5, 2>), grid, dim3(256), lds, st, a);
+        else hipLaunchKernelGGL((latent_attn_mfma_kernel<18, 8>), grid, dim3(256), lds, st, a);
+        VMX_CHECK_LAUNCH("latent_attention (matrix cores)");
+        if (a.NP > 1) {
+            hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(tokens * heads), dim3(256), 0, st, out_latent, a.part_m, a.part_l, a.part_o, sink_bf16,
+                               heads, kv_rank, a.NP);
+            VMX_CHECK_LAUNCH("latent_attention (merge)");
+        }
+        return VMX_OK;
+    }
     const size_t lds = (size_t)(kv_rank + rot_dim + 256 + 256 + 8 + 4 * kv_rank) * 4;
     dim3 grid(heads, tokens);
     if (cache_dtype == VMX_F32)
-        hipLaunchKernelGGL(latent_attn_kernel<true>, grid, dim3(256), lds, vmx_stream(stream), out_latent, q_abs, q_rot, cache, block_tables,
+        hipLaunchKernelGGL(latent_attn_kernel<true>, grid, dim3(256), lds, st, out_latent, q_abs, q_rot, cache, block_tables,
                            max_blocks_per_seq, seq_ids, positions, sink_bf16, scale, window, heads, kv_rank, rot_dim, block_size);
     else
-        hipLaunchKernelGGL(latent_attn_kernel<false>, grid, dim3(256), lds, vmx_stream(stream), out_latent, q_abs, q_rot, cache, block_tables,
+        hipLaunchKernelGGL(latent_attn_kernel<false>, grid, dim3(256), lds, st, out_latent, q_abs, q_rot, cache, block_tables,
                            max_blocks_per_seq, seq_ids, positions, sink_bf16, scale, window, heads, kv_rank, rot_dim, block_size);
     VMX_CHECK_LAUNCH("latent_attention");
     return VMX_OK;
