@@ -224,6 +224,114 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(const VmxLinear p) {
         }
 }
 
+// Up to 16 rows (decode steps, 16-row expert blocks): the product is a stream over the weights.  A workgroup owns 16 output
+// columns; its four waves split K in 128-deep blocks (wave w takes blocks w, w + 4, ...), lane (n, g) reads the 64 contiguous
+// bytes W[n][128 b + 32 g ..] of a block straight from memory, two blocks ahead of the one being multiplied, and the activation
+// fragment at the same k from the (cache-resident) rows; chunk j of both feeds MFMA step j -- the instruction only needs A and B
+// to agree on which k sits where.  The four partial tiles are added in wave order through LDS.
+__global__ __launch_bounds__(256) void linear_skinny_kernel(const VmxLinear p) {
+    __shared__ float red[3][64][4];
+    __shared__ int64_t rows[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
+    const int m0 = blockIdx.y * 16, n0 = blockIdx.x * 16, z = blockIdx.z;
+    if (p.total_rows && m0 >= *p.total_rows) return;
+    const uint16_t *W = p.W + z * p.w_bs;
+    if (p.block_expert) W += (int64_t)p.block_expert[m0 / p.block_rows] * p.expert_stride;
+    if (tid < 16) rows[tid] = linear_src_row(p, m0 + tid);
+    __syncthreads();
+    const int64_t ar = rows[fl];
+    const int n = min(n0 + fl, p.N - 1);
+    const uint16_t *wrow = W + (int64_t)n * p.w_sn;
+    const int64_t a_at = z * p.a_bs + (ar < 0 ? 0 : ar) * p.lda;
+    const int nblk = (p.K + 127) >> 7;
+    auto load_w = [&](int b, uint4 (&w)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int k = 128 * b + 32 * fg + 8 * j;
+            w[j] = k < p.K ? *reinterpret_cast<const uint4 *>(wrow + k) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto load_a = [&](int b, uint4 (&a)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int k = 128 * b + 32 * fg + 8 * j;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (ar >= 0 && k < p.K) {
+                if (p.a_f32) {
+                    const float *src = (const float *)p.A + a_at + k;
+                    const float4 f0 = *reinterpret_cast<const float4 *>(src), f1 = *reinterpret_cast<const float4 *>(src + 4);
+                    const float f[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
+                    v = vmx_pack16x8<false>(f);
+                } else {
+                    v = *reinterpret_cast<const uint4 *>((const uint16_t *)p.A + a_at + k);
+                }
+            }
+            a[j] = v;
+        }
+    };
+    vmx_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    uint4 w0[4], w1[4], a0[4], a1[4];
+    int b = wave;
+    if (b < nblk) { load_w(b, w0); load_a(b, a0); }
+    if (b + 4 < nblk) { load_w(b + 4, w1); load_a(b + 4, a1); }
+    for (; b < nblk; b += 8) {
+        uint4 wc[4], ac[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) wc[j] = w0[j], ac[j] = a0[j];
+        if (b + 8 < nblk) { load_w(b + 8, w0); load_a(b + 8, a0); }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, ac[j]), __builtin_bit_cast(vmx_bf16x8, wc[j]), acc, 0, 0, 0);
+        if (b + 4 < nblk) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) wc[j] = w1[j], ac[j] = a1[j];
+            if (b + 12 < nblk) { load_w(b + 12, w1); load_a(b + 12, a1); }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, ac[j]), __builtin_bit_cast(vmx_bf16x8, wc[j]), acc, 0, 0, 0);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wave - 1][lane][r] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float v = ((acc[r] + red[0][lane][r]) + red[1][lane][r]) + red[2][lane][r];
+            const int ml = 4 * fg + r, m = m0 + ml;
+            if (m < p.M && !(p.row_ids && rows[ml] < 0) && n0 + fl < p.N) linear_store(p, z, m, n0 + fl, v);
+        }
+    }
+}
+
+// A few output columns in true f32 (router logits): one workgroup per row and group of 16 columns; a thread walks its k with
+// stride 256 over all 16 weight rows, then lanes, then waves are added in a fixed order.  Every row count takes this kernel, so
+// a row's logits have the same bits in a prompt and in a decode step.
+__global__ __launch_bounds__(256) void linear_fewcols_f32_kernel(const VmxLinear p) {
+    __shared__ float red[4][16];
+    const int m = blockIdx.x, n0 = blockIdx.y * 16, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.f;
+    for (int k = tid; k < p.K; k += 256) {
+        const float x = ld_act(p.A, p.a_f32, (int64_t)m * p.lda + k);
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int n = min(n0 + e, p.N - 1);
+            acc[e] = fmaf(x, vmx_bf16_to_f32(p.W[(int64_t)n * p.w_sn + k]), acc[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        const float v = vmx_wave_sum(acc[e]);
+        if (lane == 0) red[wave][e] = v;
+    }
+    __syncthreads();
+    if (tid < 16 && n0 + tid < p.N) linear_store(p, 0, m, n0 + tid, (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]));
+}
+
 }  // namespace
 
 int vmx_linear_launch(const VmxLinear &p, hipStream_t st) {
@@ -234,13 +342,25 @@ int vmx_linear_launch(const VmxLinear &p, hipStream_t st) {
     VMX_REQUIRE(!p.block_expert || (p.total_rows && (p.block_rows == 16 || p.block_rows == 64)), "linear: expert blocks are 16 or 64 rows");
     VMX_REQUIRE(!p.row_ids || p.row_div >= 1, "linear: row_div must be positive");
     if (p.M == 0) return VMX_OK;
+    const bool plain = !p.row_ids && !p.block_expert && p.batch == 1 && p.w_sk == 1;
+    if (p.exact && plain && p.N <= 256) {
+        hipLaunchKernelGGL(linear_fewcols_f32_kernel, dim3(p.M, (p.N + 15) / 16), dim3(256), 0, st, p);
+        VMX_CHECK_LAUNCH("linear (few columns)");
+        return VMX_OK;
+    }
     const int bm = p.block_expert ? p.block_rows : (p.M <= 16 ? 16 : 64);
     dim3 grid((p.N + 63) / 64, (p.M + bm - 1) / bm, p.batch);
     if (p.exact) {
         if (bm == 16) hipLaunchKernelGGL(linear_fma_kernel<16>, grid, dim3(256), 0, st, p);
         else hipLaunchKernelGGL(linear_fma_kernel<64>, grid, dim3(256), 0, st, p);
     } else {
-        if (bm == 16) hipLaunchKernelGGL(linear_mfma_kernel<16>, grid, dim3(256), 0, st, p);
+        // 16-byte loads straight from the operands: whole 8-element chunks, aligned rows
+        const bool direct = p.w_sk == 1 && p.K % 8 == 0 && p.w_sn % 8 == 0 && p.lda % 8 == 0 && p.a_bs % 8 == 0 && p.w_bs % 8 == 0 &&
+                            p.expert_stride % 8 == 0 && ((uintptr_t)p.W & 15) == 0 && ((uintptr_t)p.A & 31) == 0;
+        if (bm == 16 && direct) {
+            grid.x = (p.N + 15) / 16;
+            hipLaunchKernelGGL(linear_skinny_kernel, grid, dim3(256), 0, st, p);
+        } else if (bm == 16) hipLaunchKernelGGL(linear_mfma_kernel<16>, grid, dim3(256), 0, st, p);
         else hipLaunchKernelGGL(linear_mfma_kernel<64>, grid, dim3(256), 0, st, p);
     }
     VMX_CHECK_LAUNCH("linear");
