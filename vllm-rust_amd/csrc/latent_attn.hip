@@ -389,24 +389,27 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
     }
 }
 
-// out[t, h] = sum_p e^(m_p - M) O_p / (sum_p e^(m_p - M) l_p + e^(sink - M)), M = max(sink, max_p m_p)
+// out[t, h] = sum_p e^(m_p - M) O_p / (sum_p e^(m_p - M) l_p + e^(sink - M)), M = max(sink, max_p m_p); NP <= 64.
+// Wave 0 turns the partitions' (m, l) into one weight each (one round trip to memory), then every thread sums its dimensions.
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(float *__restrict__ out, const float *__restrict__ part_m,
                                                                  const float *__restrict__ part_l, const float *__restrict__ part_o,
                                                                  const uint16_t *__restrict__ sink, int H, int R, int NP) {
+    __shared__ float wgt[64];
     const int64_t th = blockIdx.x;
-    const float sk = sink ? vmx_bf16_to_f32(sink[th % H]) : -FLT_MAX;
-    float M = sk;
-    for (int p = 0; p < NP; p++) M = fmaxf(M, part_m[th * NP + p]);
-    float den = sink ? expf(sk - M) : 0.f;
-    for (int p = 0; p < NP; p++) den += expf(part_m[th * NP + p] - M) * part_l[th * NP + p];
-    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    if (threadIdx.x < 64) {
+        const int p = threadIdx.x;
+        const float sk = sink ? vmx_bf16_to_f32(sink[th % H]) : -FLT_MAX;
+        const float m = p < NP ? part_m[th * NP + p] : -FLT_MAX, l = p < NP ? part_l[th * NP + p] : 0.f;
+        const float M = vmx_wave_max(fmaxf(l > 0.f ? m : -FLT_MAX, sk));
+        const float e = l > 0.f ? expf(m - M) : 0.f;
+        const float den = vmx_wave_sum(e * l) + (sink ? expf(sk - M) : 0.f);
+        wgt[p] = den > 0.f ? e / den : 0.f;
+    }
+    __syncthreads();
     for (int d = threadIdx.x; d < R; d += 256) {
         float v = 0.f;
-        for (int p = 0; p < NP; p++) {
-            const float l = part_l[th * NP + p];
-            if (l > 0.f) v = fmaf(expf(part_m[th * NP + p] - M), part_o[(th * NP + p) * R + d], v);
-        }
-        out[th * R + d] = v * inv;
+        for (int p = 0; p < NP; p++) v = fmaf(wgt[p], part_o[(th * NP + p) * R + d], v);
+        out[th * R + d] = v;
     }
 }
 
