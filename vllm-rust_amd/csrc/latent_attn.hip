@@ -186,9 +186,9 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float *__restrict__ ou
 //                 bf16) stay in registers, key fragments come straight from the cache rows; v_mfma_f32_16x16x32_bf16 leaves lane
 //                 (g, n) the scores of rows 4 g .. 4 g + 3 against key n, so a row's maximum and sum are DPP reductions over 16 lanes
 //                 plus one exchange between the four waves through LDS;
-//   O += P C      the tile's latents are staged TRANSPOSED in LDS ([latent dim][key], lane = key while staging, so the 2-byte
-//                 writes of a wave fall into consecutive banks) and wave w owns a quarter of the latent dimensions; P goes through
-//                 LDS as a bf16 pair hi + lo (two products), which keeps the softmax weights at f32 precision.
+//   O += P C      the key fragments a wave already holds are also written TRANSPOSED into LDS ([latent dim][key]; the cache is read
+//                 once per tile), and wave w owns a quarter of the latent dimensions of the output; P goes through LDS as a bf16
+//                 pair hi + lo (two products), which keeps the softmax weights at f32 precision.
 // A tile whose tokens belong to several sequences (decode steps of models with fewer than 16 heads) is processed once per
 // sequence with the other rows masked.  blockIdx.y splits the key range into partitions for launches with few row tiles; their
 // (max, sum, O) triples are merged, with the sink, by latent_attn_merge_kernel.
@@ -273,21 +273,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
                 sl[tid] = j <= hi ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
             }
             __syncthreads();
-            // latents of the tile, transposed: lane = key, wave w takes the 8-wide dimension chunks w, w + 4, ...
-            {
-                const int slot = sl[lane];
-                for (int dc = wave; dc < (R >> 3); dc += 4) {
-                    uint4 v = make_uint4(0, 0, 0, 0);
-                    if (slot >= 0) v = *reinterpret_cast<const uint4 *>(a.cache + (int64_t)slot * RW + 8 * dc);
-                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        CT[(8 * dc + 2 * e) * LA_LD + lane] = (uint16_t)(w4[e] & 0xFFFFu);
-                        CT[(8 * dc + 2 * e + 1) * LA_LD + lane] = (uint16_t)(w4[e] >> 16);
-                    }
-                }
-            }
-            // scores of this wave's 16 keys
+            // this wave's 16 keys: lane (n, g) reads the 16-byte chunks 32 s + 8 g of key n's cache row.  They are the B operand of
+            // the score product and, for the latent part of the row, what the transposed tile needs: each chunk is also written to
+            // CT[latent dim][key], so the cache is read once per tile.
             vmx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
             {
                 const int slot = sl[16 * wave + fl];
@@ -297,6 +285,18 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
                     const int k = 32 * s + 8 * fg;
                     kf[s] = make_uint4(0, 0, 0, 0);
                     if (s < ksteps && slot >= 0 && k < RW) kf[s] = *reinterpret_cast<const uint4 *>(a.cache + (int64_t)slot * RW + k);
+                }
+#pragma unroll
+                for (int s = 0; s < KSMAX; s++) {
+                    const int k = 32 * s + 8 * fg;
+                    if (s < ksteps && k < R) {
+                        const uint32_t w4[4] = {kf[s].x, kf[s].y, kf[s].z, kf[s].w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            CT[(k + 2 * e) * LA_LD + 16 * wave + fl] = (uint16_t)(w4[e] & 0xFFFFu);
+                            CT[(k + 2 * e + 1) * LA_LD + 16 * wave + fl] = (uint16_t)(w4[e] >> 16);
+                        }
+                    }
                 }
 #pragma unroll
                 for (int s = 0; s < KSMAX; s++)
