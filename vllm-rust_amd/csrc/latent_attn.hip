@@ -265,14 +265,18 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
         vmx_f32x4 acc[DTW];
 #pragma unroll
         for (int d = 0; d < DTW; d++) acc[d] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
+        // cache rows of a tile's keys: looked up one tile ahead, so the block table's latency is not on the tile's critical path
+        auto key_slot = [&](int kt) {
+            const int j = lo + LA_KT * kt + tid;
+            return (tid < LA_KT && kt < kt_end && j <= hi) ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
+        };
+        int next_slot = key_slot(kt_begin);
         for (int kt = kt_begin; kt < kt_end; kt++) {
             const int kbase = lo + LA_KT * kt;
-            __syncthreads();   // the previous tile's CT / P have been read
-            if (tid < LA_KT) {
-                const int j = kbase + tid;
-                sl[tid] = j <= hi ? bt[j / a.block_size] * a.block_size + j % a.block_size : -1;
-            }
+            __syncthreads();   // the previous tile's CT / P / slots have been read
+            if (tid < LA_KT) sl[tid] = next_slot;
             __syncthreads();
+            next_slot = key_slot(kt + 1);
             // this wave's 16 keys: lane (n, g) reads the 16-byte chunks 32 s + 8 g of key n's cache row.  They are the B operand of
             // the score product and, for the latent part of the row, what the transposed tile needs: each chunk is also written to
             // CT[latent dim][key], so the cache is read once per tile.
