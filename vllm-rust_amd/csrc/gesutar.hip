@@ -56,7 +56,7 @@ struct vmx_gesutar {
     Buf embed, bigram, final_norm, head;
     std::vector<std::string> missing;
     // step workspaces, sized for max_tokens
-    Buf x, h, fused, qabs, qrot, olat, attn, attn_ws, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
+    Buf x, h, fused, qabs, qrot, olat, attn, attn_ws, argmax_keys, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
     int sorted_cap = 0;
     bool f32() const { return cfg.dtype == VMX_F32; }
     size_t esz() const { return f32() ? 4 : 2; }
@@ -82,17 +82,44 @@ __global__ __launch_bounds__(256) void embed_bigram_kernel(float *__restrict__ x
     }
 }
 
-// out[r] = x[rows ? rows[r] : r] / sqrt(mean(x^2) + eps) * w, f32 statistics; out in f32 or bf16
+// out[r] = x[rows ? rows[r] : r] / sqrt(mean(x^2) + eps) * w, f32 statistics; out in f32 or bf16.  Rows up to 4096 wide stay
+// in registers between the statistic and the scaling (one trip to memory), wider rows are read twice.
 __global__ __launch_bounds__(256) void rms_norm_f32in_kernel(void *__restrict__ out, int out_f32, const float *__restrict__ x,
                                                               const int32_t *__restrict__ rows, const uint16_t *__restrict__ w, int width,
                                                               float eps) {
     __shared__ float red[4];
     const int r = blockIdx.x;
     const float *src = x + (int64_t)(rows ? rows[r] : r) * width;
+    constexpr int PT = 16;
+    float xv[PT], wv[PT];
+    const bool held = width <= 256 * PT;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < width; i += 256) ss += src[i] * src[i];
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < PT; u++) {
+            const int i = threadIdx.x + 256 * u;
+            xv[u] = i < width ? src[i] : 0.f;
+            wv[u] = i < width ? vmx_bf16_to_f32(w[i]) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < PT; u++) ss += xv[u] * xv[u];   // same order as the strided loop below
+    } else {
+        for (int i = threadIdx.x; i < width; i += 256) ss += src[i] * src[i];
+    }
     ss = vmx_block_sum_256(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < PT; u++) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < width) {
+                const float v = xv[u] * inv * wv[u];
+                if (out_f32) ((float *)out)[(int64_t)r * width + i] = v;
+                else ((uint16_t *)out)[(int64_t)r * width + i] = vmx_f32_to_bf16(v);
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < width; i += 256) {
         const float v = src[i] * inv * vmx_bf16_to_f32(w[i]);
         if (out_f32) ((float *)out)[(int64_t)r * width + i] = v;
@@ -122,29 +149,45 @@ __global__ __launch_bounds__(256) void moe_combine_f32_kernel(float *__restrict_
     x[(int64_t)t * width + i] += acc;
 }
 
-__global__ __launch_bounds__(256) void argmax_f32_kernel(int32_t *__restrict__ out, const float *__restrict__ logits, int vocab) {
-    __shared__ float bv[4];
-    __shared__ int bi[4];
-    const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float v = -FLT_MAX;
-    int ix = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += 256) {
-        const float f = logits[(int64_t)r * vocab + i];
-        if (f > v) { v = f; ix = i; }
-    }
+// Greedy ids in two launches: chunk winners as keys (order-preserving value bits | inverted index, so the largest key is the
+// largest value with the smallest index), then the winner of a row's keys.
+__device__ __forceinline__ unsigned long long argmax_key(float v, int i) {
+    uint32_t b = __float_as_uint(v);
+    b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return ((unsigned long long)b << 32) | (uint32_t)(0x7fffffff - i);
+}
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-        const float ov = vmx_lane_xor_m(v, off);
-        const int oi = vmx_lane_xor_m(ix, off);
-        if (ov > v || (ov == v && oi < ix)) { v = ov; ix = oi; }
+        const unsigned long long o = __shfl_xor(k, off, 64);
+        k = o > k ? o : k;
     }
-    if (lane == 0) { bv[wave] = v; bi[wave] = ix; }
+    return k;
+}
+constexpr int ARGMAX_CHUNK = 1024;
+__global__ __launch_bounds__(256) void argmax_f32_partial_kernel(unsigned long long *__restrict__ keys, const float *__restrict__ logits,
+                                                                  int vocab, int chunks) {
+    __shared__ unsigned long long red[4];
+    const int r = blockIdx.y, c = blockIdx.x;
+    unsigned long long best = 0;
+    for (int i = c * ARGMAX_CHUNK + threadIdx.x; i < min(vocab, (c + 1) * ARGMAX_CHUNK); i += 256) {
+        const unsigned long long k = argmax_key(logits[(int64_t)r * vocab + i], i);
+        best = k > best ? k : best;
+    }
+    best = wave_max_u64(best);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w2 = 1; w2 < 4; w2++)
-            if (bv[w2] > v || (bv[w2] == v && bi[w2] < ix)) { v = bv[w2]; ix = bi[w2]; }
-        out[r] = ix == 0x7fffffff ? 0 : ix;
+        for (int w2 = 1; w2 < 4; w2++) best = red[w2] > best ? red[w2] : best;
+        keys[(int64_t)r * chunks + c] = best;
     }
+}
+__global__ __launch_bounds__(64) void argmax_f32_final_kernel(int32_t *__restrict__ out, const unsigned long long *__restrict__ keys, int chunks) {
+    const int r = blockIdx.x;
+    unsigned long long best = 0;
+    for (int c = threadIdx.x; c < chunks; c += 64) best = keys[(int64_t)r * chunks + c] > best ? keys[(int64_t)r * chunks + c] : best;
+    best = wave_max_u64(best);
+    if (threadIdx.x == 0) out[r] = best ? 0x7fffffff - (int)(uint32_t)(best & 0xffffffffu) : 0;
 }
 
 __global__ __launch_bounds__(256) void zero_f32_kernel(float *__restrict__ p, int64_t n) {
@@ -278,6 +321,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     GA(m->olat, T * hr * 4);
     GA(m->attn_ws, (size_t)24576 * (maxr + 2) * 4);   // key partitions of launches with few rows: tokens x heads x partitions < 24576
     GA(m->attn, T * hv * m->esz());
+    GA(m->argmax_keys, T * ((size_t)c.vocab / ARGMAX_CHUNK + 1) * 8);
     GA(m->rlogits, T * ne * 4);
     GA(m->topw, (pairs + 1) * 4);
     GA(m->topi, (pairs + 1) * 4);
@@ -305,7 +349,7 @@ extern "C" void vmx_gesutar_destroy(vmx_gesutar *m) {
         for (Buf *b : {&L.norm1, &L.norm2, &L.wfused, &L.dkv_norm, &L.uk, &L.uv, &L.sink, &L.wo, &L.router, &L.eup, &L.edown, &L.sup, &L.sdown,
                        &L.inv_freq, &L.cache})
             b->release();
-    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->attn_ws, &m->rlogits,
+    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->attn_ws, &m->argmax_keys, &m->rlogits,
                    &m->topw, &m->topi, &m->sorted, &m->blk_expert, &m->total, &m->inv, &m->act, &m->ydown, &m->sact, &m->sout, &m->hsel})
         b->release();
     delete m;
@@ -526,7 +570,10 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         hd.M = num_logit_rows, hd.N = c.vocab, hd.K = W, hd.exact = f32;
         if (int rc = vmx_linear_launch(hd, st)) return rc;
         if (greedy_ids) {
-            hipLaunchKernelGGL(argmax_f32_kernel, dim3(num_logit_rows), dim3(256), 0, st, greedy_ids, lg, c.vocab);
+            const int chunks = (c.vocab + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+            hipLaunchKernelGGL(argmax_f32_partial_kernel, dim3(chunks, num_logit_rows), dim3(256), 0, st, m->argmax_keys.as<unsigned long long>(), lg,
+                               c.vocab, chunks);
+            hipLaunchKernelGGL(argmax_f32_final_kernel, dim3(num_logit_rows), dim3(64), 0, st, greedy_ids, m->argmax_keys.as<unsigned long long>(), chunks);
             VMX_CHECK_LAUNCH("gesutar argmax");
         }
     }

@@ -71,6 +71,22 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void *__restric
     }
 }
 
+// (value, index) of the wave's largest value, ties to the smaller index; every lane ends with the same pair.  The six exchange
+// steps are spelled out so that each is a DPP / permlane operation with a compile-time pattern.
+template <int M> __device__ __forceinline__ void argmax_step(float &bv, int &bi) {
+    const float ov = vmx_lane_xor<M>(bv);
+    const int oi = vmx_lane_xor<M>(bi);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+}
+__device__ __forceinline__ void wave_argmax(float &bv, int &bi) {
+    argmax_step<32>(bv, bi);
+    argmax_step<16>(bv, bi);
+    argmax_step<8>(bv, bi);
+    argmax_step<4>(bv, bi);
+    argmax_step<2>(bv, bi);
+    argmax_step<1>(bv, bi);
+}
+
 // Router with group-limited selection: softmax over all experts; the experts form `groups` equal runs of neighbours, a group's
 // score is its largest probability, and only experts of the `keep` best groups can be chosen; then k rounds of argmax (ties ->
 // smaller index) over what is left.  Weights: the chosen probabilities divided by (their sum + 1e-20), times `scale`.
@@ -123,12 +139,7 @@ __global__ __launch_bounds__(256) void grouped_topk_router_kernel(const float *_
                 const int g = lane + 64 * j;
                 if (g < groups && gv[j] > bv) { bv = gv[j]; bi = g; }
             }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                const float ov = vmx_lane_xor_m(bv, off);
-                const int oi = vmx_lane_xor_m(bi, off);
-                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-            }
+            wave_argmax(bv, bi);
 #pragma unroll
             for (int j = 0; j < 4; j++)
                 if (lane + 64 * j == bi) { gv[j] = -FLT_MAX; ok[wave][bi] = 1; }
@@ -149,12 +160,7 @@ __global__ __launch_bounds__(256) void grouped_topk_router_kernel(const float *_
             const int e = lane + 64 * j;
             if (e < E && v[j] > bv) { bv = v[j]; bi = e; }
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = vmx_lane_xor_m(bv, off);
-            const int oi = vmx_lane_xor_m(bi, off);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-        }
+        wave_argmax(bv, bi);
         if (lane == 0) { w_out[(int64_t)t * k + ki] = bv; id_out[(int64_t)t * k + ki] = bi; }
         selected += bv;
 #pragma unroll
