@@ -172,7 +172,7 @@ def _attention_ref(torch, q_abs, q_rot, rows, window, sink, scale):
 
 
 @pytest.mark.parametrize("window,use_sink,R,rd,bs", [(9, True, 24, 6, 4), (0, False, 70, 0, 16), (300, True, 130, 16, 8), (1, True, 8, 2, 3),
-                                                     (70, True, 96, 32, 16), (0, True, 40, 8, 4), (129, False, 512, 64, 16), (64, True, 136, 0, 8)])
+                                                     (70, True, 88, 24, 16), (0, True, 40, 8, 4), (129, False, 512, 64, 16), (64, True, 136, 0, 8)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_latent_attention_op(gpu, window, use_sink, R, rd, bs, dtype):
     vmx, torch = gpu
