@@ -351,6 +351,28 @@ def test_unequal_batch_against_each_alone(gpu, dtype):
     model.close()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_batches_on_both_sides_of_the_expert_sort(gpu, dtype):
+    """Decode steps of 2, 8 and 12 sequences: up to 16 (token, slot) pairs run their experts unsorted (a pair is its own row
+    block), more are sorted into expert blocks; both give the oracle's rows."""
+    from tests import gesutar_oracle as orc
+    vmx, torch = gpu
+    spec = small_spec()
+    model, eng, w = build(spec, dtype)
+    for nseq in (2, 8, 12):
+        full = [tokens_for(spec, 3 + i % 4, 60 + i, w, extra=2) for i in range(nseq)]
+        want = [orc.forward(spec, w, f).numpy() for f in full]
+        eng.step([((nseq, i), f[:-2], []) for i, f in enumerate(full)])
+        for s in (2, 1):
+            lg, _, _ = eng.step([((nseq, i), [f[-s]], [0]) for i, f in enumerate(full)])
+            lg = lg.cpu().numpy()
+            for i, f in enumerate(full):
+                assert rel_err(lg[i:i + 1], want[i][len(f) - s:len(f) - s + 1]) <= TOL[dtype], f"{nseq} sequences, request {i}"
+        for i in range(nseq):
+            eng.finish((nseq, i))
+    model.close()
+
+
 def test_blocks_freed_and_used_again(gpu):
     """A second request gets the blocks a finished one gave back (and in another order); two requests that grow in turns own
     interleaved blocks.  Results equal those on an untouched engine."""

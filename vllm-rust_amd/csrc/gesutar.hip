@@ -43,7 +43,7 @@ struct Buf {
 
 struct Layer {
     vmx_gesutar_layer_config c;
-    Buf norm1, norm2, wfused, dkv_norm, uk, uv, sink, wo, router, eup, edown, sup, sdown, inv_freq, cache;
+    Buf norm1, norm2, wfused, dkv_norm, uk, uk_t, uv, sink, wo, router, eup, edown, sup, sdown, inv_freq, cache;
     int q_off = 0, dkv_off = 0, g_off = 0, nf = 0;
     std::vector<std::string> missing;   // tensor names not loaded yet
 };
@@ -56,7 +56,7 @@ struct vmx_gesutar {
     Buf embed, bigram, final_norm, head;
     std::vector<std::string> missing;
     // step workspaces, sized for max_tokens
-    Buf x, h, fused, qabs, qrot, olat, attn, attn_ws, argmax_keys, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
+    Buf x, h, fused, qabs, qrot, olat, attn, attn_ws, argmax_keys, few_pairs, rlogits, topw, topi, sorted, blk_expert, total, inv, act, ydown, sact, sout, hsel;
     int sorted_cap = 0;
     bool f32() const { return cfg.dtype == VMX_F32; }
     size_t esz() const { return f32() ? 4 : 2; }
@@ -165,6 +165,7 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k)
     return k;
 }
 constexpr int ARGMAX_CHUNK = 1024;
+constexpr int FEW_PAIRS = 16;   // most (token, slot) pairs of a step that runs its experts unsorted
 __global__ __launch_bounds__(256) void argmax_f32_partial_kernel(unsigned long long *__restrict__ keys, const float *__restrict__ logits,
                                                                   int vocab, int chunks) {
     __shared__ unsigned long long red[4];
@@ -192,6 +193,16 @@ __global__ __launch_bounds__(64) void argmax_f32_final_kernel(int32_t *__restric
 
 __global__ __launch_bounds__(256) void zero_f32_kernel(float *__restrict__ p, int64_t n) {
     for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
+}
+
+// out[h][r][d] = in[h][d][r]: the key up-projection as [head][latent][dim], so that qa_h = U_h^T q_h reads its weights along k
+__global__ __launch_bounds__(256) void transpose_heads_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ in, int H, int D, int R) {
+    const int64_t n = (int64_t)H * D * R;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int64_t h = i / ((int64_t)D * R), rem = i % ((int64_t)D * R);
+        const int r = (int)(rem / D), d = (int)(rem % D);
+        out[i] = in[(h * D + d) * R + r];
+    }
 }
 
 int upload(Buf &b, size_t offset, const void *data, size_t bytes, hipStream_t st) {
@@ -253,6 +264,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
         GA(L.wfused, (size_t)L.nf * W * 2);
         GA(L.dkv_norm, (size_t)lc.kv_rank * 2);
         GA(L.uk, (size_t)lc.heads * lc.dim * lc.kv_rank * 2);
+        GA(L.uk_t, (size_t)lc.heads * lc.dim * lc.kv_rank * 2);
         GA(L.uv, (size_t)lc.heads * lc.vdim * lc.kv_rank * 2);
         GA(L.sink, (size_t)lc.heads * 2);
         GA(L.wo, W * ng * 2);
@@ -292,7 +304,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
             }
             ne = std::max(ne, (size_t)lc.experts);
             pairs = std::max(pairs, T * lc.top);
-            cap = std::max(cap, T * lc.top + (size_t)lc.experts * 63);
+            cap = std::max(cap, std::max(T * lc.top + (size_t)lc.experts * 63, (size_t)FEW_PAIRS * 16));
             eff = std::max(eff, (size_t)lc.expert_ff);
             sff = std::max(sff, (size_t)lc.shared_ff);
         } else if (lc.mlp != VMX_MLP_NONE) {
@@ -322,6 +334,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     GA(m->attn_ws, (size_t)24576 * (maxr + 2) * 4);   // key partitions of launches with few rows: tokens x heads x partitions < 24576
     GA(m->attn, T * hv * m->esz());
     GA(m->argmax_keys, T * ((size_t)c.vocab / ARGMAX_CHUNK + 1) * 8);
+    GA(m->few_pairs, (size_t)(2 * FEW_PAIRS * 16 + FEW_PAIRS + 1) * 4);
     GA(m->rlogits, T * ne * 4);
     GA(m->topw, (pairs + 1) * 4);
     GA(m->topi, (pairs + 1) * 4);
@@ -334,6 +347,20 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     GA(m->sact, T * (sff + 1) * m->esz());
     GA(m->sout, T * W * 4);
 #undef GA
+    if (!rc) {
+        // decode steps with a handful of (token, slot) pairs skip the sort: pair p is its own 16-row block (row 16 p)
+        std::vector<int32_t> fp(2 * FEW_PAIRS * 16 + FEW_PAIRS + 1);
+        for (int i = 0; i < FEW_PAIRS * 16; i++) {
+            fp[i] = i % 16 == 0 ? i / 16 : 0x7fffffff;                        // gathered rows of the up product: pair index or padding
+            fp[FEW_PAIRS * 16 + i] = i % 16 == 0 ? i : 0x7fffffff;            // rows of the down product: themselves or padding
+        }
+        for (int p = 0; p < FEW_PAIRS; p++) fp[2 * FEW_PAIRS * 16 + p] = 16 * p;   // where pair p's result lies
+        fp[2 * FEW_PAIRS * 16 + FEW_PAIRS] = 0x7fffffff;                       // "total rows": never cuts
+        if (hipMemcpy(m->few_pairs.p, fp.data(), fp.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
+            vmx_set_error("gesutar_create: upload failed");
+            rc = VMX_ELAUNCH;
+        }
+    }
     m->sorted_cap = (int)cap;
     if (rc) {
         vmx_gesutar_destroy(m);
@@ -346,10 +373,10 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
 extern "C" void vmx_gesutar_destroy(vmx_gesutar *m) {
     if (!m) return;
     for (Layer &L : m->layers)
-        for (Buf *b : {&L.norm1, &L.norm2, &L.wfused, &L.dkv_norm, &L.uk, &L.uv, &L.sink, &L.wo, &L.router, &L.eup, &L.edown, &L.sup, &L.sdown,
+        for (Buf *b : {&L.norm1, &L.norm2, &L.wfused, &L.dkv_norm, &L.uk, &L.uk_t, &L.uv, &L.sink, &L.wo, &L.router, &L.eup, &L.edown, &L.sup, &L.sdown,
                        &L.inv_freq, &L.cache})
             b->release();
-    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->attn_ws, &m->argmax_keys, &m->rlogits,
+    for (Buf *b : {&m->embed, &m->bigram, &m->final_norm, &m->head, &m->x, &m->h, &m->fused, &m->qabs, &m->qrot, &m->olat, &m->attn, &m->attn_ws, &m->argmax_keys, &m->few_pairs, &m->rlogits,
                    &m->topw, &m->topi, &m->sorted, &m->blk_expert, &m->total, &m->inv, &m->act, &m->ydown, &m->sact, &m->sout, &m->hsel})
         b->release();
     delete m;
@@ -407,8 +434,16 @@ extern "C" int vmx_gesutar_load_tensor(vmx_gesutar *m, const char *name, const v
     }
     VMX_REQUIRE(dst, "gesutar_load_tensor: unknown tensor `%s`", name);
     VMX_REQUIRE(bytes == need, "gesutar_load_tensor: `%s`: expected %zu bytes of bf16, got %zu", name, need, bytes);
-    if (bytes > 0)
+    if (bytes > 0) {
         if (int rc = upload(*dst, off, data, bytes, st)) return rc;
+        if (n.size() > 7 && n.compare(n.size() - 7, 7, ".mix.uk") == 0) {
+            Layer &L = m->layers[atoi(n.substr(1).c_str())];
+            hipLaunchKernelGGL(transpose_heads_kernel, dim3(512), dim3(256), 0, st, L.uk_t.as<uint16_t>(), L.uk.as<uint16_t>(), L.c.heads, L.c.dim,
+                               L.c.kv_rank);
+            VMX_CHECK_LAUNCH("gesutar transpose");
+            VMX_CHECK_HIP(hipStreamSynchronize(st));
+        }
+    }
     erase_name(*missing, n);
     return VMX_OK;
 }
@@ -466,7 +501,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         if (dim > 0) {   // qa_h = U_h^T q_h: per head, [T, dim] x [dim, R]
             VmxLinear a;
             a.A = m->fused.as<float>() + L.q_off, a.a_f32 = 1, a.lda = L.nf, a.a_bs = dim + rd;
-            a.W = L.uk.as<uint16_t>(), a.w_sn = 1, a.w_sk = R, a.w_bs = (int64_t)dim * R;
+            a.W = L.uk_t.as<uint16_t>(), a.w_sn = dim, a.w_sk = 1, a.w_bs = (int64_t)dim * R;
             a.C = m->qabs.p, a.c_f32 = 1, a.ldc = (int64_t)H * R, a.c_bs = R;
             a.M = T, a.N = R, a.K = dim, a.batch = H, a.exact = f32;
             if (int rc = vmx_linear_launch(a, st)) return rc;
@@ -507,31 +542,42 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
             r.C = m->rlogits.p, r.c_f32 = 1, r.ldc = E;
             r.M = T, r.N = E, r.K = W, r.exact = 1;
             if (int rc = vmx_linear_launch(r, st)) return rc;
+            // logits and routing stay two launches: one workgroup per token doing both walks K once per 16 experts in sequence
+            // (21.5 us at one row of 2048 against 10.3 + 5.7 us for the pair)
             if (int rc = vmx_grouped_topk_router(m->rlogits.as<float>(), m->topw.as<float>(), m->topi.as<int32_t>(), T, E, k, lc.groups,
                                                  lc.keep_groups, lc.router_scale, st))
                 return rc;
-            const int br = pairs >= 32 * E ? 64 : 16;
-            const int cap = pairs + E * (br - 1);
-            if (int rc = vmx_moe_align_block_size(m->topi.as<int32_t>(), m->sorted.as<int32_t>(), m->blk_expert.as<int32_t>(),
-                                                  m->total.as<int32_t>(), pairs, E, br, cap, st))
-                return rc;
-            hipLaunchKernelGGL(moe_inverse_kernel, dim3((cap + 255) / 256), dim3(256), 0, st, m->inv.as<int32_t>(), m->sorted.as<int32_t>(),
-                               m->total.as<int32_t>(), pairs);
-            VMX_CHECK_LAUNCH("gesutar moe inverse");
-            VmxLinear u;   // act = relu(W_up[e] h)^2 over the sorted pairs
+            const bool few = pairs <= FEW_PAIRS;   // every pair its own block: no sort, an expert's weights are read once per pair
+            const int br = few ? 16 : (pairs >= 32 * E ? 64 : 16);
+            const int cap = few ? pairs * 16 : pairs + E * (br - 1);
+            const int32_t *fp = m->few_pairs.as<int32_t>();
+            const int32_t *up_rows = few ? fp : m->sorted.as<int32_t>(), *down_rows = few ? fp + FEW_PAIRS * 16 : nullptr;
+            const int32_t *blk = few ? m->topi.as<int32_t>() : m->blk_expert.as<int32_t>();
+            const int32_t *total = few ? fp + 2 * FEW_PAIRS * 16 + FEW_PAIRS : m->total.as<int32_t>();
+            const int32_t *inv = few ? fp + 2 * FEW_PAIRS * 16 : m->inv.as<int32_t>();
+            if (!few) {
+                if (int rc = vmx_moe_align_block_size(m->topi.as<int32_t>(), m->sorted.as<int32_t>(), m->blk_expert.as<int32_t>(),
+                                                      m->total.as<int32_t>(), pairs, E, br, cap, st))
+                    return rc;
+                hipLaunchKernelGGL(moe_inverse_kernel, dim3((cap + 255) / 256), dim3(256), 0, st, m->inv.as<int32_t>(), m->sorted.as<int32_t>(),
+                                   m->total.as<int32_t>(), pairs);
+                VMX_CHECK_LAUNCH("gesutar moe inverse");
+            }
+            VmxLinear u;   // act = relu(W_up[e] h)^2 over the pairs' rows
             u.A = m->h.p, u.a_f32 = f32, u.lda = W;
             u.W = L.eup.as<uint16_t>(), u.w_sn = W, u.w_sk = 1;
             u.C = m->act.p, u.c_f32 = f32, u.ldc = ff;
             u.M = cap, u.N = ff, u.K = W, u.exact = f32, u.epilogue = VMX_EP_RELU2;
-            u.row_ids = m->sorted.as<int32_t>(), u.row_div = k, u.row_limit = pairs;
-            u.block_expert = m->blk_expert.as<int32_t>(), u.expert_stride = (int64_t)ff * W, u.block_rows = br, u.total_rows = m->total.as<int32_t>();
+            u.row_ids = up_rows, u.row_div = k, u.row_limit = pairs;
+            u.block_expert = blk, u.expert_stride = (int64_t)ff * W, u.block_rows = br, u.total_rows = total;
             if (int rc = vmx_linear_launch(u, st)) return rc;
             VmxLinear d;   // y = W_down[e] act
             d.A = m->act.p, d.a_f32 = f32, d.lda = ff;
             d.W = L.edown.as<uint16_t>(), d.w_sn = ff, d.w_sk = 1;
             d.C = m->ydown.p, d.c_f32 = 1, d.ldc = W;
             d.M = cap, d.N = W, d.K = ff, d.exact = f32;
-            d.block_expert = m->blk_expert.as<int32_t>(), d.expert_stride = (int64_t)ff * W, d.block_rows = br, d.total_rows = m->total.as<int32_t>();
+            d.row_ids = down_rows, d.row_div = 1, d.row_limit = cap;
+            d.block_expert = blk, d.expert_stride = (int64_t)ff * W, d.block_rows = br, d.total_rows = total;
             if (int rc = vmx_linear_launch(d, st)) return rc;
             const float *shared = nullptr;
             if (lc.shared_ff > 0) {
@@ -549,8 +595,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
                 if (int rc = vmx_linear_launch(sd, st)) return rc;
                 shared = m->sout.as<float>();
             }
-            hipLaunchKernelGGL(moe_combine_f32_kernel, dim3((W + 255) / 256, T), dim3(256), 0, st, x, m->ydown.as<float>(), m->inv.as<int32_t>(),
-                               m->topw.as<float>(), k, shared, W);
+            hipLaunchKernelGGL(moe_combine_f32_kernel, dim3((W + 255) / 256, T), dim3(256), 0, st, x, m->ydown.as<float>(), inv, m->topw.as<float>(), k, shared, W);
             VMX_CHECK_LAUNCH("gesutar moe combine");
         }
         if (layer_trace)
