@@ -537,3 +537,20 @@ def test_trace_replay_tool(gpu, tmp_path):
         s2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(1, spec.vocab)
         assert not (out / "1.f32").exists()
         assert rel_err(s0, np.stack([wa[0], wa[6], wb[3]])) <= TOL[dtype] and rel_err(s2, wa[8:9]) <= TOL[dtype]
+
+
+def test_engine_serves_the_qwen3_executor_too(gpu):
+    """The same Engine (block manager, scheduler, packed steps) over the Qwen3 executor through its adapter: greedy ids of three
+    prompts generated together equal each prompt generated alone on an untouched engine."""
+    vmx, torch = gpu
+    from vllm_rust_amd.engine import Engine, PackedQwen3, SamplingParams
+    from vllm_rust_amd.qwen3 import QuantizedQwen3ForCausalLM, Qwen3Spec
+    spec = Qwen3Spec(hidden_size=256, num_layers=2, num_heads=4, num_kv_heads=2, head_dim=64, intermediate_size=512, vocab_size=1000,
+                     max_position=256, num_blocks=24, max_batch=4, max_seq_len=128, max_prefill_tokens=64)
+    model = QuantizedQwen3ForCausalLM(spec)
+    model.load_synthetic(seed=2)
+    prompts = [np.random.default_rng(70 + i).integers(0, 1000, n).tolist() for i, n in enumerate([5, 17, 1])]
+    together = Engine(PackedQwen3(model)).generate(prompts, SamplingParams(max_new_tokens=6))
+    alone = [Engine(PackedQwen3(model)).generate([p], SamplingParams(max_new_tokens=6))[0] for p in prompts]
+    assert together == alone and all(len(o) == 6 for o in together)
+    model.close()
