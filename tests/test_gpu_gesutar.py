@@ -554,3 +554,46 @@ def test_engine_serves_the_qwen3_executor_too(gpu):
     alone = [Engine(PackedQwen3(model)).generate([p], SamplingParams(max_new_tokens=6))[0] for p in prompts]
     assert together == alone and all(len(o) == 6 for o in together)
     model.close()
+
+
+def _random_spec(seed):
+    """A configuration drawn at random: per-layer sizes, windows, rotation, router shape; some layers without feed-forward."""
+    from vllm_rust_amd.gesutar import GesutarLayerSpec, GesutarSpec
+    r = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(r.integers(0, len(xs)))]
+    step = pick(8, 8, 2)                                      # multiples of 8 take the matrix-core attention, others the vector form
+    layers = []
+    for li in range(int(r.integers(1, 4))):
+        dim, rd = pick((0, 2), (1, 1), (2, 1), (3, 2), (1, 0), (5, 3))
+        dim, rd = dim * step, rd * step
+        rot_dims = 0 if rd == 0 else pick(rd, rd, max(2, rd // 2 // 2 * 2))
+        groups = pick(1, 2, 3)
+        per = pick(1, 2, 4)
+        keep = int(r.integers(1, groups + 1))
+        moe = li == 0 or r.random() < 0.7
+        layers.append(GesutarLayerSpec(heads=int(r.integers(1, 10)), dim=dim, rot_dim=rd, vdim=pick(1, 3, 5) * step, kv_rank=pick(1, 2, 5, 9, 17) * step,
+                                       window=pick(1, 2, 7, 16, 33, 65, 500), rot_dims=rot_dims, rot_base=pick(100.0, 10000.0, 5e5),
+                                       scale=pick(0.1, 0.25, 0.5), mlp="moe" if moe else None, experts=groups * per,
+                                       top=int(r.integers(1, keep * per + 1)), groups=groups, keep_groups=keep, expert_ff=pick(6, 16, 40),
+                                       shared_ff=pick(0, 8, 24), router_scale=pick(1.0, 2.5)))
+    return GesutarSpec(vocab=pick(17, 100, 257), width=pick(24, 40, 64, 72), layers=layers, norm_eps=pick(1e-5, 1e-6), embed_scale=pick(1.0, 4.0),
+                       bigram_buckets=pick(1, 31, 509), bigram_mul_prev=pick(1, 31, 65537), bigram_mul_cur=pick(1, 7))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(gpu, seed):
+    """Ten configurations drawn at random, each a 45-token prompt and 25 decoded tokens in both modes against the oracle."""
+    from tests import gesutar_oracle as orc
+    vmx, torch = gpu
+    spec = _random_spec(seed)
+    for dtype in ("float32", "bfloat16"):
+        model, eng, w = build(spec, dtype, seed=seed, block_size=int(np.random.default_rng(seed).integers(1, 9)), num_blocks=96)
+        toks = tokens_for(spec, 70, 100 + seed, w if dtype == "bfloat16" else None)
+        want = orc.forward(spec, w, toks).numpy()
+        lg, _, _ = eng.step([("r", toks[:45], list(range(45)))])
+        rows = [lg.cpu().numpy()]
+        for t in toks[45:]:
+            lg, _, _ = eng.step([("r", [t], [0])])
+            rows.append(lg.cpu().numpy())
+        assert rel_err(np.concatenate(rows), want) <= TOL[dtype] * (1 if dtype == "float32" else 1.5), f"{dtype}: {spec}"
+        model.close()

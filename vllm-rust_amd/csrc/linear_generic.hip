@@ -6,9 +6,12 @@
 //   * gathered activation rows and per-row-block weight matrices (experts of a mixture whose (token, slot) pairs were sorted into
 //     blocks by vmx_moe_align_block_size);
 //   * epilogues: plain store, squared ReLU, accumulate into an f32 residual stream, multiply by sigmoid(gate).
-// Two kernels: `linear_fma_kernel` multiplies in true f32 on the vector ALU (the 32-bit mode of a model, and every product that
-// must stay in 32 bits such as a router), `linear_mfma_kernel` rounds the activations to bf16 and runs v_mfma_f32_16x16x32_bf16.
-// A row's result never depends on the other rows of the call: a row is summed in the same order whatever M is.
+// Kernels: `linear_mfma_kernel` (64-row tiles for prompts and 64-row expert blocks; a staged 16-row form for shapes the streaming
+// kernel does not take) and `linear_skinny_kernel` (up to 16 rows: decode steps and 16-row expert blocks, weights streamed once)
+// round the activations to bf16 and run v_mfma_f32_16x16x32_bf16; `linear_fma_kernel` multiplies in true f32 on the vector ALU
+// (the 32-bit mode of a model), `linear_fewcols_f32_kernel` does the same for a few output columns (router logits) with one
+// kernel for every row count.  A row's result never depends on the other rows of the call: within a kernel a row is summed in
+// the same order whatever M is; between the streaming and the tiled kernels the order differs (rounding-level differences).
 #include "vmx_kernels.h"
 
 namespace {

@@ -10,7 +10,6 @@ token ids come out.
 from __future__ import annotations
 
 import collections
-import ctypes as C
 import dataclasses
 
 import numpy as np

@@ -143,22 +143,19 @@ def synthetic_weights(spec: GesutarSpec, seed: int = 0, device="cpu") -> dict:
     """Seeded random-init checkpoint of the architecture (bf16 tensors on `device`): matrices ~ 1 / sqrt(in), norm weights
     around 1, sinks around 0, so that activations stay O(1) through the stack."""
     g = torch.Generator(device=device).manual_seed(seed)
-    _randn = torch.randn
 
-    class torch_:   # every draw on the generator's device
-        @staticmethod
-        def randn(shape, generator):
-            return _randn(shape, generator=generator, device=device)
+    def randn(shape):
+        return torch.randn(shape, generator=g, device=device)
     ck = {}
     for name, shape in spec.tensor_shapes().items():
         if name.endswith("norm1") or name.endswith("norm2") or name.endswith(".norm"):
-            t = 1.0 + 0.1 * torch_.randn(shape, generator=g)
+            t = 1.0 + 0.1 * randn(shape)
         elif name.endswith("sink"):
-            t = 0.5 * torch_.randn(shape, generator=g)
+            t = 0.5 * randn(shape)
         elif name in ("embed", "bigram"):
-            t = torch_.randn(shape, generator=g) * (0.5 if name == "bigram" else 1.0 / max(spec.embed_scale, 1e-6))
+            t = randn(shape) * (0.5 if name == "bigram" else 1.0 / max(spec.embed_scale, 1e-6))
         else:
-            t = torch_.randn(shape, generator=g) / math.sqrt(shape[-1])
+            t = randn(shape) / math.sqrt(shape[-1])
         ck[name] = t.to(torch.bfloat16)
     return ck
 
