@@ -916,7 +916,9 @@ def main():
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
     ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
-                         "their own block), so that a kernel trace of the run holds that workload's launches only")
+                         "their own block), so that a kernel trace of the run holds that workload's launches only; gesutar = the Gesutar "
+                         "executor (latent attention + grouped-router MoE, bf16) at two layer sizes beside the bf16 dense Qwen3 executor at "
+                         "equal size: prompt tok/s and decode tok/s at 1 and 16 sequences (not part of the default run)")
     ap.add_argument("--tp", action="store_true", help="accepted for compatibility: with --gpus N > 1 the tensor-parallel job is the default")
     ap.add_argument("--replicas", action="store_true",
                     help="with --gpus N > 1: N independent replicas as the primary (weak scaling, no collective) instead of ONE model "
