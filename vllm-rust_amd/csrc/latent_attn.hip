@@ -186,9 +186,10 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float *__restrict__ ou
 //                 bf16) stay in registers, key fragments come straight from the cache rows; v_mfma_f32_16x16x32_bf16 leaves lane
 //                 (g, n) the scores of rows 4 g .. 4 g + 3 against key n, so a row's maximum and sum are DPP reductions over 16 lanes
 //                 plus one exchange between the four waves through LDS;
-//   O += P C      the key fragments a wave already holds are also written TRANSPOSED into LDS ([latent dim][key]; the cache is read
-//                 once per tile), and wave w owns a quarter of the latent dimensions of the output; P goes through LDS as a bf16
-//                 pair hi + lo (two products), which keeps the softmax weights at f32 precision.
+//   O += P C      the key fragments a wave already holds also go row-major into LDS (one 16-byte write per fragment; the cache is
+//                 read once per tile) and come back as C^T through the transposing LDS read (ds_read_b64_tr_b16); wave w owns a
+//                 quarter of the latent dimensions of the output; P goes through LDS as a bf16 pair hi + lo (two products), which
+//                 keeps the softmax weights at f32 precision.
 // A tile whose tokens belong to several sequences (decode steps of models with fewer than 16 heads) is processed once per
 // sequence with the other rows masked.  blockIdx.y splits the key range into partitions for launches with few row tiles; their
 // (max, sum, O) triples are merged, with the sink, by latent_attn_merge_kernel.
@@ -203,14 +204,18 @@ struct LatentAttnArgs {
     int max_blocks, window, T, H, R, rd, block_size, HPT, TPT, NHG, NP;
 };
 
-constexpr int LA_KT = 64, LA_LD = LA_KT + 8;
+constexpr int LA_KT = 64, LA_LD = LA_KT + 8;   // keys per tile; row stride of the P tiles
+constexpr int LA_PAD = 32;                    // the row-major latent tile pads its rows by 64 bytes: four consecutive rows, four bank groups
+typedef short la_s16x4 __attribute__((ext_vector_type(4)));
+typedef short la_s16x8 __attribute__((ext_vector_type(8)));
 
 template <int KSMAX, int DTW>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnArgs a) {
     extern __shared__ __align__(16) unsigned char la_smem[];
     const int R = a.R, RW = a.R + a.rd;
-    uint16_t *CT = reinterpret_cast<uint16_t *>(la_smem);            // [R][LA_LD]
-    uint16_t *Phi = CT + (size_t)R * LA_LD;                           // [16][LA_LD]
+    const int ROWE = R + LA_PAD;
+    uint16_t *KT = reinterpret_cast<uint16_t *>(la_smem);            // [LA_KT][R + LA_PAD]: the tile's latents, row-major
+    uint16_t *Phi = KT + (size_t)LA_KT * ROWE;                        // [16][LA_LD]
     uint16_t *Plo = Phi + 16 * LA_LD;                                 // [16][LA_LD]
     float *red_max = reinterpret_cast<float *>(Plo + 16 * LA_LD);     // [4][16]
     float *red_sum = red_max + 64;                                    // [4][16]
@@ -273,13 +278,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
         int next_slot = key_slot(kt_begin);
         for (int kt = kt_begin; kt < kt_end; kt++) {
             const int kbase = lo + LA_KT * kt;
-            __syncthreads();   // the previous tile's CT / P / slots have been read
+            __syncthreads();   // the previous tile's latents / P / slots have been read
             if (tid < LA_KT) sl[tid] = next_slot;
             __syncthreads();
             next_slot = key_slot(kt + 1);
             // this wave's 16 keys: lane (n, g) reads the 16-byte chunks 32 s + 8 g of key n's cache row.  They are the B operand of
-            // the score product and, for the latent part of the row, what the transposed tile needs: each chunk is also written to
-            // CT[latent dim][key], so the cache is read once per tile.
+            // the score product and, for the latent part of the row, the tile of the value product: each chunk is also written to
+            // KT[key][latent dim], so the cache is read once per tile.
             vmx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
             {
                 const int slot = sl[16 * wave + fl];
@@ -293,14 +298,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
 #pragma unroll
                 for (int s = 0; s < KSMAX; s++) {
                     const int k = 32 * s + 8 * fg;
-                    if (s < ksteps && k < R) {
-                        const uint32_t w4[4] = {kf[s].x, kf[s].y, kf[s].z, kf[s].w};
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            CT[(k + 2 * e) * LA_LD + 16 * wave + fl] = (uint16_t)(w4[e] & 0xFFFFu);
-                            CT[(k + 2 * e + 1) * LA_LD + 16 * wave + fl] = (uint16_t)(w4[e] >> 16);
-                        }
-                    }
+                    if (s < ksteps && k < R) *reinterpret_cast<uint4 *>(KT + (16 * wave + fl) * ROWE + k) = kf[s];
                 }
 #pragma unroll
                 for (int s = 0; s < KSMAX; s++)
@@ -351,8 +349,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const LatentAttnA
 #pragma unroll
                 for (int d = 0; d < DTW; d++) {
                     if (d < dt_per_wave && dt0 + d < dtiles) {
-                        const int dim = min(16 * (dt0 + d) + fl, R - 1);
-                        const uint4 cf = *reinterpret_cast<const uint4 *>(CT + dim * LA_LD + 32 * ks + 8 * fg);
+                        // B operand = C^T: the transposing LDS read hands lane n the values of column 16 dt + n for the four rows
+                        // (keys) its 16-lane group addressed; two reads give the eight keys 32 ks + 8 g .. + 7 of this lane's k slots
+                        const uint16_t *src = KT + (32 * ks + 8 * fg + (fl >> 2)) * ROWE + 16 * (dt0 + d) + 4 * (fl & 3);
+                        const la_s16x4 c0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((la_s16x4 __attribute__((address_space(3))) *)src);
+                        const la_s16x4 c1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((la_s16x4 __attribute__((address_space(3))) *)(src + 4 * ROWE));
+                        const la_s16x8 cf = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
                         acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, ah), __builtin_bit_cast(vmx_bf16x8, cf), acc[d], 0, 0,
                                                                          0);
                         acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, al), __builtin_bit_cast(vmx_bf16x8, cf), acc[d], 0, 0,
@@ -486,7 +488,7 @@ extern "C" int vmx_latent_attention(float *out_latent, const float *q_abs, const
         a.part_m = (float *)workspace;
         a.part_l = a.part_m + (size_t)tokens * heads * a.NP;
         a.part_o = a.part_l + (size_t)tokens * heads * a.NP;
-        const size_t lds = ((size_t)kv_rank * LA_LD + 2 * 16 * LA_LD) * 2 + (64 + 64) * 4 + 64 * 4;
+        const size_t lds = ((size_t)LA_KT * (kv_rank + LA_PAD) + 2 * 16 * LA_LD) * 2 + (64 + 64) * 4 + 64 * 4;
         dim3 grid((unsigned)(((tokens + a.TPT - 1) / a.TPT) * a.NHG), a.NP);
         const bool small = RW <= 160 && kv_rank <= 128;
         const void *fn = small ? (const void *)latent_attn_mfma_kernel<5, 2> : (const void *)latent_attn_mfma_kernel<18, 8>;
