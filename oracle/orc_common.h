@@ -2,7 +2,7 @@
  * CPU oracle -- TEST INFRASTRUCTURE ONLY.
  *
  * A plain-C restatement of the reference's CPU algorithms for the quantized
- * inference hot path.  It is the checker for the HIP kernels: only tests/,
+ * inference hot path.  It is what the HIP kernels are compared against: only tests/,
  * __graft_entry__.smoke() and bench.py's cpu_baseline leg may load it.  The
  * product library (libvmx.so) never links or calls anything in this directory.
  *
