@@ -597,3 +597,30 @@ def test_random_configurations(gpu, seed):
             rows.append(lg.cpu().numpy())
         assert rel_err(np.concatenate(rows), want) <= TOL[dtype] * (1 if dtype == "float32" else 1.5), f"{dtype}: {spec}"
         model.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_windows_over_several_key_tiles(gpu, dtype):
+    """A 230-token prompt and 40 decoded tokens through layers whose windows (150 and 70 tokens) span several 64-key tiles of the
+    matrix-core attention, so that prompts walk many tiles and decode steps split their keys over partitions; far keys matter
+    because the sinks are low and the scores sharp."""
+    from tests import gesutar_oracle as orc
+    from vllm_rust_amd.gesutar import GesutarLayerSpec
+    vmx, torch = gpu
+    base = dict(heads=4, dim=16, rot_dim=8, vdim=16, kv_rank=32, rot_dims=8, scale=1.5, experts=2, top=2, groups=1, keep_groups=1,
+                expert_ff=16, shared_ff=8)      # every expert is chosen: no router decision that rounding could flip
+    spec = small_spec(layers=[GesutarLayerSpec(window=150, **base), GesutarLayerSpec(window=70, **base)])
+
+    def low_sinks(ck):
+        for i in range(2):
+            ck[f"l{i}.mix.sink"].fill_(-6.0)
+    model, eng, w = build(spec, dtype, tweak=low_sinks, block_size=16, num_blocks=40, max_tokens=512)
+    toks = tokens_for(spec, 270, 9, w if dtype == "bfloat16" else None)
+    want = orc.forward(spec, w, toks).numpy()
+    lg, _, _ = eng.step([("s", toks[:230], list(range(230)))])
+    rows = [lg.cpu().numpy()]
+    for t in toks[230:]:
+        lg, _, _ = eng.step([("s", [t], [0])])
+        rows.append(lg.cpu().numpy())
+    assert rel_err(np.concatenate(rows), want) <= TOL[dtype] * (1 if dtype == "float32" else 1.5)
+    model.close()
