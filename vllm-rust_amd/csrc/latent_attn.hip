@@ -441,16 +441,16 @@ extern "C" int vmx_latent_kv_prepare(const float *fused, int64_t ld_fused, int q
     return VMX_OK;
 }
 
-// Partition count of the matrix-core form for a launch (host arithmetic only): 1 when there are enough row tiles to fill the
-// device, else enough key partitions to give every compute unit a workgroup.
+// Partition count of the matrix-core form for a launch (host arithmetic only): one workgroup fits a compute unit at the largest
+// latent size, so the launch is given at most one workgroup per compute unit -- row tiles x partitions <= compute units -- and a
+// launch with that many row tiles or more is not split at all.
 static int latent_attn_partitions(int tokens, int heads, int window, int max_blocks_per_seq, int block_size) {
     const int hpt = heads < 16 ? heads : 16, tpt = 16 / hpt, nhg = (heads + hpt - 1) / hpt;
     const int64_t tiles = (int64_t)((tokens + tpt - 1) / tpt) * nhg;
     int64_t max_keys = (int64_t)max_blocks_per_seq * block_size;
     if (window > 0 && window < max_keys) max_keys = window;
     const int64_t key_tiles = max_keys / LA_KT + 1;
-    if (tiles >= 512) return 1;
-    int64_t np = (1024 + tiles - 1) / tiles;
+    int64_t np = vmx_num_cus() / tiles;
     if (np > key_tiles) np = key_tiles;
     if (np > 64) np = 64;
     return np < 1 ? 1 : (int)np;
