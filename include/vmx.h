@@ -1020,6 +1020,94 @@ int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const int32_t *pr
                         const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids, float *layer_trace,
                         void *stream);
 
+/* ------------------------------------------------- window attention, short convolution, gated delta rule, Gupuvik executor */
+
+/* The step's key and value rows (f32, row strides ldk / ldv) into cache rows slots[t] of two caches with rows of k_width and
+ * v_width elements (negative slot: not stored).  cache_dtype VMX_F32 / VMX_BF16. */
+int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *v, int64_t ldv, const int32_t *slots, void *k_cache, void *v_cache,
+                           int cache_dtype, int tokens, int k_width, int v_width, void *stream);
+/* Grouped-query attention of packed tokens over paged caches (rows [kv_heads * dim] and [kv_heads * vdim], found through
+ * block_tables[seq_ids[t]]): score = (q . k) * scale * head_temp[h] (bf16 per head, NULL: 1), then softcap * tanh(score / softcap)
+ * (softcap 0: none), softmax over the keys j <= i = positions[t] with i - j < window (0: all) or j < keep_first, weighted sum of
+ * the values, times sigmoid(gate[t * ldgate + h]) (NULL: none).  q f32 rows of heads * dim at stride ldq; out [tokens, heads * vdim]
+ * f32 or bf16.  No rotation.  Scores and softmax in f32. */
+int vmx_window_attention(void *out, int out_dtype, const float *q, int64_t ldq, const void *k_cache, const void *v_cache, int cache_dtype,
+                         const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
+                         const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale, float softcap, int window,
+                         int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim, int block_size, void *stream);
+
+/* Short causal convolution over time per channel with carried state, then SiLU: y[t, c] = silu(sum_s taps[c, n - 1 - s] x[t - s, c]);
+ * inputs from before the step come from state[state_slots[seq]] ([taps - 1, channels] f32, the sequence's last inputs), inputs from
+ * before position 0 are zero.  Tokens are packed: sequence s owns rows seq_starts[s] .. seq_starts[s + 1] - 1 at consecutive
+ * positions.  The first unit_groups runs of unit_group channels are then scaled to unit vectors (x / sqrt(sum x^2 + unit_eps)), the
+ * first scaled_groups of them also multiplied by scaled_mul.  y must not alias x.  Call vmx_short_conv_state_update afterwards. */
+size_t vmx_short_conv_state_bytes(int slots, int channels, int taps);
+int vmx_short_conv_silu(const float *x, int64_t ldx, const uint16_t *taps_bf16, float *state, float *y, int64_t ldy, const int32_t *positions,
+                        const int32_t *seq_ids, const int32_t *seq_starts, const int32_t *state_slots, int tokens, int channels, int taps,
+                        int unit_group, int unit_groups, int scaled_groups, float unit_eps, float scaled_mul, void *stream);
+int vmx_short_conv_state_update(const float *x, int64_t ldx, float *state, const int32_t *positions, const int32_t *seq_starts,
+                                const int32_t *state_slots, int num_seqs, int channels, int taps, void *stream);
+/* In place: g[t, c] <- exp(-exp(A_log[c / dim]) * softplus(g[t, c] + dt_bias[c])) for c < heads * dim, beta[t, h] <- sigmoid(beta[t, h]). */
+int vmx_delta_rule_gates(float *g, int64_t ldg, const uint16_t *a_log_bf16, const uint16_t *dt_bias_bf16, float *beta, int64_t ldbeta,
+                         int tokens, int heads, int dim, void *stream);
+/* Gated delta rule per head over a matrix memory S [dim, vdim] (f32, in state[state_slots[seq]], layout private to the kernel;
+ * a sequence whose step starts at position 0 starts from zeros):  S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
+ * o_t = S^T q_t.  q, k rows of qk_heads * dim, v, o rows of heads * vdim, g rows of heads * dim, beta rows of heads; dim <= 256. */
+size_t vmx_gated_delta_rule_state_bytes(int slots, int heads, int dim, int vdim);
+int vmx_gated_delta_rule(float *o, int64_t ldo, const float *q, int64_t ldq, const float *k, int64_t ldk, const float *v, int64_t ldv,
+                         const float *g, int64_t ldg, const float *beta, int64_t ldbeta, float *state, const int32_t *positions,
+                         const int32_t *seq_starts, const int32_t *state_slots, int num_seqs, int heads, int qk_heads, int dim, int vdim,
+                         void *stream);
+/* y[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * w (bf16 [vdim], shared by the heads) * sigmoid(gate[t, h]) (NULL: none). */
+int vmx_head_rms_gate(void *y, int y_dtype, const float *o, int64_t ldo, const uint16_t *w_bf16, const float *gate, int64_t ldgate, float eps,
+                      int tokens, int heads, int vdim, void *stream);
+
+#define VMX_MIXER_WINDOW_ATTENTION 1
+#define VMX_MIXER_CHANNEL_DELTA 2
+#define VMX_MLP_DENSE_GELU 2
+#define VMX_MLP_GLU_MOE 3
+
+/* One layer of a Gupuvik model.  The layer is parallel: h = norm(x) (one gain for the row), x += sigmoid(R1 h + r1) * mixer(h)
+ * + sigmoid(R2 h + r2) * ff(h). */
+typedef struct vmx_gupuvik_layer_config {
+    int mixer;                  /* VMX_MIXER_WINDOW_ATTENTION or VMX_MIXER_CHANNEL_DELTA */
+    int heads, kv_heads, dim, vdim;   /* query (value) heads, key heads, key size, value size */
+    int window, keep_first;     /* attention: window 0 = every earlier key */
+    float scale, softcap;       /* attention: score scale; softcap 0 = none */
+    int kv_from;                /* attention: layer whose key/value cache this layer reads instead of its own (-1: own) */
+    int conv_taps, decay_rank, gate_rank;   /* channel delta: taps of the short convolution, ranks of the decay and gate projections */
+    int mlp;                    /* VMX_MLP_NONE, VMX_MLP_DENSE_GELU or VMX_MLP_GLU_MOE */
+    int ff;                     /* dense feed-forward width */
+    int experts, top, expert_ff;
+} vmx_gupuvik_layer_config;
+
+typedef struct vmx_gupuvik_config {
+    int vocab, width, num_layers;
+    float norm_eps;
+    double embed_scale;
+    int dtype;                  /* VMX_BF16: bf16 operands and cache; VMX_F32: everything in f32 */
+    int block_size, num_blocks; /* paged key/value cache: rows per block, blocks per layer */
+    int max_tokens, max_seqs;   /* most tokens / sequences of one forward call */
+    int state_slots;            /* recurrent-state slots (one per live sequence) */
+} vmx_gupuvik_config;
+
+typedef struct vmx_gupuvik vmx_gupuvik;
+int vmx_gupuvik_create(const vmx_gupuvik_config *cfg, const vmx_gupuvik_layer_config *layers, vmx_gupuvik **out);
+void vmx_gupuvik_destroy(vmx_gupuvik *m);
+/* One checkpoint tensor under its name in the file: "embed", "head", "final.norm", "l<i>.norm1", "l<i>.rg1|rg2" (+ ".b"),
+ * attention "l<i>.mix.q|k|v" (+ ".b"), "mix.temp|g|o", channel delta "l<i>.mix.q|k|v" (+ ".conv"), "mix.b|A_log|norm|a1|a2|dt_bias|g1|g2|o",
+ * "l<i>.mlp.up|down", "l<i>.mlp.router", "l<i>.mlp.e<j>.gate|up|down": bf16, matrices [out, in]; host or device memory. */
+int vmx_gupuvik_load_tensor(vmx_gupuvik *m, const char *name, const void *data, size_t bytes, void *stream);
+int vmx_gupuvik_missing_tensors(const vmx_gupuvik *m);
+/* One step over packed tokens (device i32 arrays): token t has id tokens[t], position positions[t], cache row slots[t] and
+ * belongs to sequence seq_ids[t]; sequence s owns the rows seq_starts[s] .. seq_starts[s + 1] - 1 (consecutive positions), the
+ * blocks block_tables[s] and the recurrent-state slot state_slots[s].  A sequence whose first row is at position 0 starts with
+ * empty state.  Outputs as vmx_gesutar_forward. */
+int vmx_gupuvik_forward(vmx_gupuvik *m, const int32_t *tokens, const int32_t *positions, const int32_t *slots, const int32_t *seq_ids,
+                        int num_tokens, const int32_t *block_tables, int num_seqs, int max_blocks_per_seq, const int32_t *seq_starts,
+                        const int32_t *state_slots, const int32_t *logit_rows, int num_logit_rows, float *logits, int32_t *greedy_ids,
+                        float *layer_trace, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -221,6 +221,20 @@ _SIGS = {
     "vmx_gesutar_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
     "vmx_gesutar_missing_tensors": (_i, [_p]),
     "vmx_gesutar_forward": (_i, [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _i, _p, _p, _p, _p]),
+    "vmx_kv_cache_write_f32": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "vmx_window_attention": (_i, [_p, _i, _p, _i64, _p, _p, _i, _p, _i, _p, _p, _p, _p, _i64, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "vmx_short_conv_state_bytes": (_sz, [_i, _i, _i]),
+    "vmx_short_conv_silu": (_i, [_p, _i64, _p, _p, _p, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p]),
+    "vmx_short_conv_state_update": (_i, [_p, _i64, _p, _p, _p, _p, _i, _i, _i, _p]),
+    "vmx_delta_rule_gates": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _i, _p]),
+    "vmx_gated_delta_rule_state_bytes": (_sz, [_i, _i, _i, _i]),
+    "vmx_gated_delta_rule": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "vmx_head_rms_gate": (_i, [_p, _i, _p, _i64, _p, _p, _i64, _f, _i, _i, _i, _p]),
+    "vmx_gupuvik_create": (_i, [_p, _p, _p]),
+    "vmx_gupuvik_destroy": (None, [_p]),
+    "vmx_gupuvik_load_tensor": (_i, [_p, C.c_char_p, _p, _sz, _p]),
+    "vmx_gupuvik_missing_tensors": (_i, [_p]),
+    "vmx_gupuvik_forward": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
 }
 
 
@@ -267,6 +281,23 @@ class GesutarConfig(C.Structure):
         ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("embed_scale", C.c_double), ("bigram_buckets", _i),
         ("bigram_mul_prev", _i), ("bigram_mul_cur", _i), ("dtype", _i), ("block_size", _i), ("num_blocks", _i), ("max_tokens", _i),
         ("max_seqs", _i),
+    ]
+
+
+class GupuvikLayerConfig(C.Structure):
+    """struct vmx_gupuvik_layer_config (include/vmx.h)."""
+    _fields_ = [
+        ("mixer", _i), ("heads", _i), ("kv_heads", _i), ("dim", _i), ("vdim", _i), ("window", _i), ("keep_first", _i), ("scale", _f),
+        ("softcap", _f), ("kv_from", _i), ("conv_taps", _i), ("decay_rank", _i), ("gate_rank", _i), ("mlp", _i), ("ff", _i), ("experts", _i),
+        ("top", _i), ("expert_ff", _i),
+    ]
+
+
+class GupuvikConfig(C.Structure):
+    """struct vmx_gupuvik_config (include/vmx.h)."""
+    _fields_ = [
+        ("vocab", _i), ("width", _i), ("num_layers", _i), ("norm_eps", _f), ("embed_scale", C.c_double), ("dtype", _i), ("block_size", _i),
+        ("num_blocks", _i), ("max_tokens", _i), ("max_seqs", _i), ("state_slots", _i),
     ]
 
 

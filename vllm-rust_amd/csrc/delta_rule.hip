@@ -1,0 +1,286 @@
+// Gated delta rule with one decay per key channel, as a recurrent token mixer over packed steps, and the short causal
+// convolution in front of it.  Both carry state from step to step in a SLOT per sequence (the caller's state-slot manager hands
+// them out); a sequence whose step starts at position 0 starts from zeros whatever its slot held before.
+//
+// Short convolution (vmx_short_conv_silu): y[t, c] = silu(sum_s taps[c, n - 1 - s] * x[t - s, c]), zeros before the sequence's
+// first token.  The last n - 1 inputs of every sequence are its state [slots, n - 1, channels] (f32); inputs older than the step
+// come from there.  A group of channels (one head's query or key) may then be scaled to a unit vector, x / sqrt(sum x^2 + eps),
+// times a constant.  vmx_short_conv_state_update moves the state on after all of a step's rows were read.
+//
+// Recurrence (vmx_gated_delta_rule), per head with a matrix memory S [dim, vdim] in f32:
+//   S <- diag(g_t) S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
+// so a token reads the memory after its own write.  Query/key head of value head h: h / (heads / qk_heads).  A workgroup owns 32
+// value columns of one (sequence, head) and walks the sequence's tokens of the step in order; 8 threads share a column, each
+// holding every 8th row of S in registers, and the two column sums per token are 8-lane butterflies.  The state slot keeps S in
+// the workgroup's own register order (the layout is private to this kernel), so that loading and storing it is coalesced.
+#include "vmx_kernels.h"
+
+namespace {
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+struct ConvArgs {
+    const float *x;          // [tokens, ldx] inputs of the step, channels at column 0
+    int64_t ldx;
+    const uint16_t *taps;    // bf16 [channels, n]
+    float *state;            // [slots, n - 1, channels]
+    float *y;                // [tokens, ldy]
+    int64_t ldy;
+    const int32_t *positions, *seq_ids, *seq_starts, *state_slots;
+    int tokens, channels, n;
+    // unit-vector groups: channels [0, unit_groups * group) are groups of `group` channels; groups < scaled_groups also get `mul`
+    int group, unit_groups, scaled_groups;
+    float unit_eps, mul;
+};
+
+// one wave per (token, run of `group` channels); runs past the unit groups are plain 64-channel runs
+__global__ __launch_bounds__(256) void short_conv_silu_kernel(const ConvArgs a) {
+    const int t = blockIdx.y, lane = threadIdx.x & 63;
+    const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int unit_ch = a.unit_groups * a.group;
+    int c0, c1;
+    bool unit = false;
+    if (run < a.unit_groups) c0 = run * a.group, c1 = c0 + a.group, unit = true;
+    else c0 = unit_ch + (run - a.unit_groups) * 64, c1 = min(c0 + 64, a.channels);
+    if (c0 >= a.channels) return;
+    const int pos = a.positions[t], seq = a.seq_ids[t];
+    const int first = a.seq_starts[seq];             // packed row of the sequence's first token in this step
+    const int start = pos - (t - first);             // position of that token
+    const float *st = a.state + (int64_t)a.state_slots[seq] * (a.n - 1) * a.channels;
+    float ss = 0.f;
+    for (int c = c0 + lane; c < c1; c += 64) {
+        float acc = 0.f;
+        for (int s = a.n - 1; s >= 0; s--) {         // oldest input first
+            const int q = pos - s;
+            if (q < 0) continue;
+            const float xv = q >= start ? a.x[(int64_t)(t - s) * a.ldx + c] : st[(int64_t)(q - start + a.n - 1) * a.channels + c];
+            acc = fmaf(vmx_bf16_to_f32(a.taps[(int64_t)c * a.n + (a.n - 1 - s)]), xv, acc);
+        }
+        const float yv = silu_f(acc);
+        a.y[(int64_t)t * a.ldy + c] = yv;
+        ss = fmaf(yv, yv, ss);
+    }
+    if (unit) {
+        ss = vmx_wave_sum(ss);
+        const float f = (run < a.scaled_groups ? a.mul : 1.0f) / sqrtf(ss + a.unit_eps);
+        for (int c = c0 + lane; c < c1; c += 64) a.y[(int64_t)t * a.ldy + c] *= f;   // each lane rescales what it wrote itself
+    }
+}
+
+// state[slot] <- the last n - 1 inputs of the sequence after this step.  A thread owns one (sequence, channel) and goes through
+// the state rows in ascending order: row r takes the input of position end - (n - 1) + r, which is a row of the step or an OLDER
+// state row r + count (not overwritten yet).
+__global__ __launch_bounds__(256) void short_conv_state_kernel(const ConvArgs a, int num_seqs) {
+    const int seq = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= a.channels) return;
+    const int first = a.seq_starts[seq], count = a.seq_starts[seq + 1] - first;
+    if (count <= 0) return;
+    const int start = a.positions[first];
+    float *st = a.state + (int64_t)a.state_slots[seq] * (a.n - 1) * a.channels;
+    for (int r = 0; r < a.n - 1; r++) {
+        const int q = start + count - (a.n - 1) + r;
+        float v = 0.f;
+        if (q >= start) v = a.x[(int64_t)(first + q - start) * a.ldx + c];
+        else if (q >= 0) v = st[(int64_t)(r + count) * a.channels + c];
+        st[(int64_t)r * a.channels + c] = v;
+    }
+}
+
+// g[t, c] <- exp(-exp(A_log[c / dim]) * softplus(g[t, c] + dt_bias[c])) in place, and beta[t, h] <- sigmoid(beta[t, h]) in place
+__global__ __launch_bounds__(256) void delta_gates_kernel(float *__restrict__ g, int64_t ldg, const uint16_t *__restrict__ a_log,
+                                                           const uint16_t *__restrict__ dt_bias, float *__restrict__ beta, int64_t ldbeta,
+                                                           int heads, int dim) {
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c < heads * dim) {
+        const float rate = expf(vmx_bf16_to_f32(a_log[c / dim]));
+        const float dt = softplus_f(g[(int64_t)t * ldg + c] + vmx_bf16_to_f32(dt_bias[c]));
+        g[(int64_t)t * ldg + c] = expf(-rate * dt);
+    }
+    if (c < heads) beta[(int64_t)t * ldbeta + c] = sigmoid_f(beta[(int64_t)t * ldbeta + c]);
+}
+
+struct DeltaArgs {
+    const float *q, *k, *v, *g, *beta;       // rows of the step: q, k [qk_heads * dim], v [heads * vdim], g [heads * dim], beta [heads]
+    int64_t ldq, ldk, ldv, ldg, ldbeta;
+    float *o;                                // [tokens, heads * vdim]
+    int64_t ldo;
+    float *state;                            // [slots, heads, tiles, DPT, 256]
+    const int32_t *positions, *seq_starts, *state_slots;
+    int heads, qk_heads, dim, vdim;
+};
+
+constexpr int DR_RS = 8, DR_VT = 32, DR_CT = 8;   // row splits per column, columns per workgroup, tokens staged per round
+
+template <int DPT>
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a) {
+    constexpr int DP = DPT * DR_RS;          // padded key dimension
+    __shared__ float sq[DR_CT][DP], sk[DR_CT][DP], sg[DR_CT][DP], sv[DR_CT][DR_VT], sb[DR_CT];
+    const int seq = blockIdx.z, h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+    const int first = a.seq_starts[seq], count = a.seq_starts[seq + 1] - first;
+    if (count <= 0) return;
+    const int r = tid & (DR_RS - 1), cl = tid >> 3, c = tile * DR_VT + cl;
+    const int qh = h / (a.heads / a.qk_heads);
+    const int tiles = gridDim.x;
+    float *sp = a.state + ((((int64_t)a.state_slots[seq] * a.heads + h) * tiles + tile) * DPT) * 256 + tid;
+    float S[DPT];
+    const bool fresh = a.positions[first] == 0;
+#pragma unroll
+    for (int u = 0; u < DPT; u++) S[u] = fresh ? 0.f : sp[(int64_t)u * 256];
+    for (int t0 = 0; t0 < count; t0 += DR_CT) {
+        const int ct = min(DR_CT, count - t0);
+        __syncthreads();
+        for (int i = tid; i < ct * DP; i += 256) {
+            const int tt = i / DP, d = i % DP;
+            const int64_t row = first + t0 + tt;
+            const bool in = d < a.dim;
+            sq[tt][d] = in ? a.q[row * a.ldq + (int64_t)qh * a.dim + d] : 0.f;
+            sk[tt][d] = in ? a.k[row * a.ldk + (int64_t)qh * a.dim + d] : 0.f;
+            sg[tt][d] = in ? a.g[row * a.ldg + (int64_t)h * a.dim + d] : 1.f;
+        }
+        for (int i = tid; i < ct * DR_VT; i += 256) {
+            const int tt = i / DR_VT, cc = tile * DR_VT + i % DR_VT;
+            sv[tt][i % DR_VT] = cc < a.vdim ? a.v[(int64_t)(first + t0 + tt) * a.ldv + (int64_t)h * a.vdim + cc] : 0.f;
+        }
+        if (tid < ct) sb[tid] = a.beta[(int64_t)(first + t0 + tid) * a.ldbeta + h];
+        __syncthreads();
+        for (int tt = 0; tt < ct; tt++) {
+            float kk[DPT], part = 0.f;
+#pragma unroll
+            for (int u = 0; u < DPT; u++) {
+                kk[u] = sk[tt][r + DR_RS * u];
+                S[u] *= sg[tt][r + DR_RS * u];
+                part = fmaf(S[u], kk[u], part);
+            }
+            part += vmx_dpp<VMX_DPP_XOR1>(part);
+            part += vmx_dpp<VMX_DPP_XOR2>(part);
+            part += vmx_dpp<VMX_DPP_HALF_MIRROR>(part);
+            const float uu = sb[tt] * (sv[tt][cl] - part);
+            float po = 0.f;
+#pragma unroll
+            for (int u = 0; u < DPT; u++) {
+                S[u] = fmaf(kk[u], uu, S[u]);
+                po = fmaf(S[u], sq[tt][r + DR_RS * u], po);
+            }
+            po += vmx_dpp<VMX_DPP_XOR1>(po);
+            po += vmx_dpp<VMX_DPP_XOR2>(po);
+            po += vmx_dpp<VMX_DPP_HALF_MIRROR>(po);
+            if (r == 0 && c < a.vdim) a.o[(int64_t)(first + t0 + tt) * a.ldo + (int64_t)h * a.vdim + c] = po;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < DPT; u++) sp[(int64_t)u * 256] = S[u];
+}
+
+// y[t, h] = o[t, h] / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h]); one wave per (token, head); w bf16 [vdim] shared by heads
+__global__ __launch_bounds__(256) void head_rms_gate_kernel(void *__restrict__ y, int y_f32, const float *__restrict__ o, int64_t ldo,
+                                                             const uint16_t *__restrict__ w, const float *__restrict__ gate, int64_t ldgate,
+                                                             float eps, int rows, int heads, int vdim) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const int t = row / heads, h = row % heads;
+    const float *src = o + (int64_t)t * ldo + (int64_t)h * vdim;
+    float ss = 0.f;
+    for (int i = lane; i < vdim; i += 64) ss = fmaf(src[i], src[i], ss);
+    ss = vmx_wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+    for (int i = lane; i < vdim; i += 64) {
+        float v = src[i] * inv * vmx_bf16_to_f32(w[i]);
+        if (gate) v *= sigmoid_f(gate[(int64_t)t * ldgate + (int64_t)h * vdim + i]);
+        const int64_t at = ((int64_t)t * heads + h) * vdim + i;
+        if (y_f32) ((float *)y)[at] = v;
+        else ((uint16_t *)y)[at] = vmx_f32_to_bf16(v);
+    }
+}
+
+ConvArgs conv_args(const float *x, int64_t ldx, const uint16_t *taps, float *state, float *y, int64_t ldy, const int32_t *positions,
+                   const int32_t *seq_ids, const int32_t *seq_starts, const int32_t *state_slots, int tokens, int channels, int n, int group,
+                   int unit_groups, int scaled_groups, float unit_eps, float mul) {
+    return ConvArgs{x, ldx, taps, state, y, ldy, positions, seq_ids, seq_starts, state_slots, tokens, channels, n, group, unit_groups,
+                    scaled_groups, unit_eps, mul};
+}
+
+}  // namespace
+
+extern "C" size_t vmx_short_conv_state_bytes(int slots, int channels, int taps) {
+    return (size_t)slots * (size_t)(taps > 1 ? taps - 1 : 0) * channels * 4;
+}
+
+extern "C" int vmx_short_conv_silu(const float *x, int64_t ldx, const uint16_t *taps_bf16, float *state, float *y, int64_t ldy,
+                                   const int32_t *positions, const int32_t *seq_ids, const int32_t *seq_starts, const int32_t *state_slots,
+                                   int tokens, int channels, int taps, int unit_group, int unit_groups, int scaled_groups, float unit_eps,
+                                   float scaled_mul, void *stream) {
+    VMX_REQUIRE(x && taps_bf16 && y && positions && seq_ids && seq_starts && state_slots && (state || taps <= 1), "short_conv: null pointer");
+    VMX_REQUIRE(channels >= 1 && taps >= 1 && ldx >= channels && ldy >= channels, "short_conv: bad sizes");
+    VMX_REQUIRE(unit_groups >= 0 && scaled_groups >= 0 && scaled_groups <= unit_groups && (unit_groups == 0 || unit_group >= 1) &&
+                    (int64_t)unit_groups * unit_group <= channels,
+                "short_conv: bad unit-vector groups");
+    if (tokens <= 0) return VMX_OK;
+    const ConvArgs a = conv_args(x, ldx, taps_bf16, state, y, ldy, positions, seq_ids, seq_starts, state_slots, tokens, channels, taps, unit_group,
+                                 unit_groups, scaled_groups, unit_eps, scaled_mul);
+    const int runs = unit_groups + (channels - unit_groups * unit_group + 63) / 64;
+    hipLaunchKernelGGL(short_conv_silu_kernel, dim3((runs + 3) / 4, tokens), dim3(256), 0, vmx_stream(stream), a);
+    VMX_CHECK_LAUNCH("short_conv_silu");
+    return VMX_OK;
+}
+
+extern "C" int vmx_short_conv_state_update(const float *x, int64_t ldx, float *state, const int32_t *positions, const int32_t *seq_starts,
+                                           const int32_t *state_slots, int num_seqs, int channels, int taps, void *stream) {
+    VMX_REQUIRE(x && positions && seq_starts && state_slots && (state || taps <= 1), "short_conv_state_update: null pointer");
+    if (num_seqs <= 0 || taps <= 1) return VMX_OK;
+    const ConvArgs a = conv_args(x, ldx, nullptr, state, nullptr, 0, positions, nullptr, seq_starts, state_slots, 0, channels, taps, 1, 0, 0, 0.f, 1.f);
+    hipLaunchKernelGGL(short_conv_state_kernel, dim3((channels + 255) / 256, num_seqs), dim3(256), 0, vmx_stream(stream), a, num_seqs);
+    VMX_CHECK_LAUNCH("short_conv_state_update");
+    return VMX_OK;
+}
+
+extern "C" int vmx_delta_rule_gates(float *g, int64_t ldg, const uint16_t *a_log_bf16, const uint16_t *dt_bias_bf16, float *beta,
+                                    int64_t ldbeta, int tokens, int heads, int dim, void *stream) {
+    VMX_REQUIRE(g && a_log_bf16 && dt_bias_bf16 && beta, "delta_rule_gates: null pointer");
+    VMX_REQUIRE(heads >= 1 && dim >= 1 && ldg >= (int64_t)heads * dim && ldbeta >= heads, "delta_rule_gates: bad sizes");
+    if (tokens <= 0) return VMX_OK;
+    hipLaunchKernelGGL(delta_gates_kernel, dim3((heads * dim + 255) / 256, tokens), dim3(256), 0, vmx_stream(stream), g, ldg, a_log_bf16,
+                       dt_bias_bf16, beta, ldbeta, heads, dim);
+    VMX_CHECK_LAUNCH("delta_rule_gates");
+    return VMX_OK;
+}
+
+static int delta_dpt(int dim) { return dim <= 64 ? 8 : (dim <= 128 ? 16 : 32); }
+
+extern "C" size_t vmx_gated_delta_rule_state_bytes(int slots, int heads, int dim, int vdim) {
+    const size_t tiles = (vdim + DR_VT - 1) / DR_VT;
+    return (size_t)slots * heads * tiles * delta_dpt(dim) * 256 * 4;
+}
+
+extern "C" int vmx_gated_delta_rule(float *o, int64_t ldo, const float *q, int64_t ldq, const float *k, int64_t ldk, const float *v,
+                                    int64_t ldv, const float *g, int64_t ldg, const float *beta, int64_t ldbeta, float *state,
+                                    const int32_t *positions, const int32_t *seq_starts, const int32_t *state_slots, int num_seqs, int heads,
+                                    int qk_heads, int dim, int vdim, void *stream) {
+    VMX_REQUIRE(o && q && k && v && g && beta && state && positions && seq_starts && state_slots, "gated_delta_rule: null pointer");
+    VMX_REQUIRE(heads >= 1 && qk_heads >= 1 && heads % qk_heads == 0, "gated_delta_rule: %d heads do not share %d query/key heads evenly", heads,
+                qk_heads);
+    VMX_REQUIRE(dim >= 1 && dim <= 256 && vdim >= 1, "gated_delta_rule: key size %d outside 1..256", dim);
+    if (num_seqs <= 0) return VMX_OK;
+    const DeltaArgs a{q, k, v, g, beta, ldq, ldk, ldv, ldg, ldbeta, o, ldo, state, positions, seq_starts, state_slots, heads, qk_heads, dim, vdim};
+    const dim3 grid((vdim + DR_VT - 1) / DR_VT, heads, num_seqs), block(256);
+    hipStream_t st = vmx_stream(stream);
+    switch (delta_dpt(dim)) {
+        case 8: hipLaunchKernelGGL(gated_delta_rule_kernel<8>, grid, block, 0, st, a); break;
+        case 16: hipLaunchKernelGGL(gated_delta_rule_kernel<16>, grid, block, 0, st, a); break;
+        default: hipLaunchKernelGGL(gated_delta_rule_kernel<32>, grid, block, 0, st, a); break;
+    }
+    VMX_CHECK_LAUNCH("gated_delta_rule");
+    return VMX_OK;
+}
+
+extern "C" int vmx_head_rms_gate(void *y, int y_dtype, const float *o, int64_t ldo, const uint16_t *w_bf16, const float *gate, int64_t ldgate,
+                                 float eps, int tokens, int heads, int vdim, void *stream) {
+    VMX_REQUIRE(y && o && w_bf16, "head_rms_gate: null pointer");
+    VMX_REQUIRE(y_dtype == VMX_F32 || y_dtype == VMX_BF16, "head_rms_gate: f32 or bf16 output");
+    if (tokens <= 0) return VMX_OK;
+    hipLaunchKernelGGL(head_rms_gate_kernel, dim3((tokens * heads + 3) / 4), dim3(256), 0, vmx_stream(stream), y, y_dtype == VMX_F32, o, ldo,
+                       w_bf16, gate, ldgate, eps, tokens * heads, heads, vdim);
+    VMX_CHECK_LAUNCH("head_rms_gate");
+    return VMX_OK;
+}

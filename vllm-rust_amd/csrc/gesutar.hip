@@ -20,26 +20,7 @@
 
 namespace {
 
-struct Buf {
-    void *p = nullptr;
-    size_t bytes = 0;
-    int alloc(size_t n) {
-        release();
-        bytes = n;
-        hipError_t e = hipMalloc(&p, n ? n : 16);
-        if (e != hipSuccess) {
-            p = nullptr;
-            vmx_set_error("hipMalloc(%zu) failed: %s", n, hipGetErrorString(e));
-            return VMX_ENOMEM;
-        }
-        return VMX_OK;
-    }
-    void release() {
-        if (p) (void)hipFree(p);
-        p = nullptr;
-    }
-    template <typename T> T *as() const { return (T *)p; }
-};
+using Buf = VmxBuf;
 
 struct Layer {
     vmx_gesutar_layer_config c;
@@ -80,119 +61,6 @@ __global__ __launch_bounds__(256) void embed_bigram_kernel(float *__restrict__ x
         if (buckets > 0) v += vmx_bf16_to_f32(bigram[row * width + i]);
         x[(int64_t)t * width + i] = v;
     }
-}
-
-// out[r] = x[rows ? rows[r] : r] / sqrt(mean(x^2) + eps) * w, f32 statistics; out in f32 or bf16.  Rows up to 4096 wide stay
-// in registers between the statistic and the scaling (one trip to memory), wider rows are read twice.
-__global__ __launch_bounds__(256) void rms_norm_f32in_kernel(void *__restrict__ out, int out_f32, const float *__restrict__ x,
-                                                              const int32_t *__restrict__ rows, const uint16_t *__restrict__ w, int width,
-                                                              float eps) {
-    __shared__ float red[4];
-    const int r = blockIdx.x;
-    const float *src = x + (int64_t)(rows ? rows[r] : r) * width;
-    constexpr int PT = 16;
-    float xv[PT], wv[PT];
-    const bool held = width <= 256 * PT;
-    float ss = 0.f;
-    if (held) {
-#pragma unroll
-        for (int u = 0; u < PT; u++) {
-            const int i = threadIdx.x + 256 * u;
-            xv[u] = i < width ? src[i] : 0.f;
-            wv[u] = i < width ? vmx_bf16_to_f32(w[i]) : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < PT; u++) ss += xv[u] * xv[u];   // same order as the strided loop below
-    } else {
-        for (int i = threadIdx.x; i < width; i += 256) ss += src[i] * src[i];
-    }
-    ss = vmx_block_sum_256(ss, red);
-    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-    if (held) {
-#pragma unroll
-        for (int u = 0; u < PT; u++) {
-            const int i = threadIdx.x + 256 * u;
-            if (i < width) {
-                const float v = xv[u] * inv * wv[u];
-                if (out_f32) ((float *)out)[(int64_t)r * width + i] = v;
-                else ((uint16_t *)out)[(int64_t)r * width + i] = vmx_f32_to_bf16(v);
-            }
-        }
-        return;
-    }
-    for (int i = threadIdx.x; i < width; i += 256) {
-        const float v = src[i] * inv * vmx_bf16_to_f32(w[i]);
-        if (out_f32) ((float *)out)[(int64_t)r * width + i] = v;
-        else ((uint16_t *)out)[(int64_t)r * width + i] = vmx_f32_to_bf16(v);
-    }
-}
-
-// inv[pair] = position of the pair in the expert-sorted list
-__global__ __launch_bounds__(256) void moe_inverse_kernel(int32_t *__restrict__ inv, const int32_t *__restrict__ sorted,
-                                                           const int32_t *__restrict__ total, int numel) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < *total) {
-        const int p = sorted[i];
-        if (p >= 0 && p < numel) inv[p] = i;
-    }
-}
-
-// x[t] += sum_slot w[t, slot] * y[inv[t * k + slot]] (slot order) + shared[t]
-__global__ __launch_bounds__(256) void moe_combine_f32_kernel(float *__restrict__ x, const float *__restrict__ y,
-                                                               const int32_t *__restrict__ inv, const float *__restrict__ w, int k,
-                                                               const float *__restrict__ shared, int width) {
-    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= width) return;
-    float acc = 0.f;
-    for (int s = 0; s < k; s++) acc = fmaf(w[(int64_t)t * k + s], y[(int64_t)inv[(int64_t)t * k + s] * width + i], acc);
-    if (shared) acc += shared[(int64_t)t * width + i];
-    x[(int64_t)t * width + i] += acc;
-}
-
-// Greedy ids in two launches: chunk winners as keys (order-preserving value bits | inverted index, so the largest key is the
-// largest value with the smallest index), then the winner of a row's keys.
-__device__ __forceinline__ unsigned long long argmax_key(float v, int i) {
-    uint32_t b = __float_as_uint(v);
-    b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-    return ((unsigned long long)b << 32) | (uint32_t)(0x7fffffff - i);
-}
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const unsigned long long o = __shfl_xor(k, off, 64);
-        k = o > k ? o : k;
-    }
-    return k;
-}
-constexpr int ARGMAX_CHUNK = 1024;
-constexpr int FEW_PAIRS = 16;   // most (token, slot) pairs of a step that runs its experts unsorted
-__global__ __launch_bounds__(256) void argmax_f32_partial_kernel(unsigned long long *__restrict__ keys, const float *__restrict__ logits,
-                                                                  int vocab, int chunks) {
-    __shared__ unsigned long long red[4];
-    const int r = blockIdx.y, c = blockIdx.x;
-    unsigned long long best = 0;
-    for (int i = c * ARGMAX_CHUNK + threadIdx.x; i < min(vocab, (c + 1) * ARGMAX_CHUNK); i += 256) {
-        const unsigned long long k = argmax_key(logits[(int64_t)r * vocab + i], i);
-        best = k > best ? k : best;
-    }
-    best = wave_max_u64(best);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w2 = 1; w2 < 4; w2++) best = red[w2] > best ? red[w2] : best;
-        keys[(int64_t)r * chunks + c] = best;
-    }
-}
-__global__ __launch_bounds__(64) void argmax_f32_final_kernel(int32_t *__restrict__ out, const unsigned long long *__restrict__ keys, int chunks) {
-    const int r = blockIdx.x;
-    unsigned long long best = 0;
-    for (int c = threadIdx.x; c < chunks; c += 64) best = keys[(int64_t)r * chunks + c] > best ? keys[(int64_t)r * chunks + c] : best;
-    best = wave_max_u64(best);
-    if (threadIdx.x == 0) out[r] = best ? 0x7fffffff - (int)(uint32_t)(best & 0xffffffffu) : 0;
-}
-
-__global__ __launch_bounds__(256) void zero_f32_kernel(float *__restrict__ p, int64_t n) {
-    for (int64_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
 }
 
 // out[h][r][d] = in[h][d][r]: the key up-projection as [head][latent][dim], so that qa_h = U_h^T q_h reads its weights along k
@@ -304,7 +172,7 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
             }
             ne = std::max(ne, (size_t)lc.experts);
             pairs = std::max(pairs, T * lc.top);
-            cap = std::max(cap, std::max(T * lc.top + (size_t)lc.experts * 63, (size_t)FEW_PAIRS * 16));
+            cap = std::max(cap, std::max(T * lc.top + (size_t)lc.experts * 63, (size_t)VMX_MOE_FEW_PAIRS * 16));
             eff = std::max(eff, (size_t)lc.expert_ff);
             sff = std::max(sff, (size_t)lc.shared_ff);
         } else if (lc.mlp != VMX_MLP_NONE) {
@@ -333,8 +201,8 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
     GA(m->olat, T * hr * 4);
     GA(m->attn_ws, (size_t)24576 * (maxr + 2) * 4);   // key partitions of launches with few rows: tokens x heads x partitions < 24576
     GA(m->attn, T * hv * m->esz());
-    GA(m->argmax_keys, T * ((size_t)c.vocab / ARGMAX_CHUNK + 1) * 8);
-    GA(m->few_pairs, (size_t)(2 * FEW_PAIRS * 16 + FEW_PAIRS + 1) * 4);
+    GA(m->argmax_keys, T * ((size_t)c.vocab / VMX_ARGMAX_CHUNK + 1) * 8);
+    GA(m->few_pairs, (size_t)(2 * VMX_MOE_FEW_PAIRS * 16 + VMX_MOE_FEW_PAIRS + 1) * 4);
     GA(m->rlogits, T * ne * 4);
     GA(m->topw, (pairs + 1) * 4);
     GA(m->topi, (pairs + 1) * 4);
@@ -349,13 +217,13 @@ extern "C" int vmx_gesutar_create(const vmx_gesutar_config *cfg, const vmx_gesut
 #undef GA
     if (!rc) {
         // decode steps with a handful of (token, slot) pairs skip the sort: pair p is its own 16-row block (row 16 p)
-        std::vector<int32_t> fp(2 * FEW_PAIRS * 16 + FEW_PAIRS + 1);
-        for (int i = 0; i < FEW_PAIRS * 16; i++) {
+        std::vector<int32_t> fp(2 * VMX_MOE_FEW_PAIRS * 16 + VMX_MOE_FEW_PAIRS + 1);
+        for (int i = 0; i < VMX_MOE_FEW_PAIRS * 16; i++) {
             fp[i] = i % 16 == 0 ? i / 16 : 0x7fffffff;                        // gathered rows of the up product: pair index or padding
-            fp[FEW_PAIRS * 16 + i] = i % 16 == 0 ? i : 0x7fffffff;            // rows of the down product: themselves or padding
+            fp[VMX_MOE_FEW_PAIRS * 16 + i] = i % 16 == 0 ? i : 0x7fffffff;            // rows of the down product: themselves or padding
         }
-        for (int p = 0; p < FEW_PAIRS; p++) fp[2 * FEW_PAIRS * 16 + p] = 16 * p;   // where pair p's result lies
-        fp[2 * FEW_PAIRS * 16 + FEW_PAIRS] = 0x7fffffff;                       // "total rows": never cuts
+        for (int p = 0; p < VMX_MOE_FEW_PAIRS; p++) fp[2 * VMX_MOE_FEW_PAIRS * 16 + p] = 16 * p;   // where pair p's result lies
+        fp[2 * VMX_MOE_FEW_PAIRS * 16 + VMX_MOE_FEW_PAIRS] = 0x7fffffff;                       // "total rows": never cuts
         if (hipMemcpy(m->few_pairs.p, fp.data(), fp.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
             vmx_set_error("gesutar_create: upload failed");
             rc = VMX_ELAUNCH;
@@ -485,9 +353,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         const vmx_gesutar_layer_config &lc = L.c;
         const int H = lc.heads, R = lc.kv_rank, rd = lc.rot_dim, dim = lc.dim, vd = lc.vdim;
         // ---- mixer: latent attention
-        hipLaunchKernelGGL(rms_norm_f32in_kernel, dim3(T), dim3(256), 0, st, m->h.p, f32, x, (const int32_t *)nullptr, L.norm1.as<uint16_t>(), W,
-                           c.norm_eps);
-        VMX_CHECK_LAUNCH("gesutar norm1");
+        if (int rc = vmx_rms_norm_f32in(m->h.p, f32, x, nullptr, L.norm1.as<uint16_t>(), 0, W, c.norm_eps, T, st)) return rc;
         VmxLinear p;
         p.A = m->h.p, p.a_f32 = f32, p.lda = W;
         p.W = L.wfused.as<uint16_t>(), p.w_sn = W, p.w_sk = 1;
@@ -506,8 +372,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
             a.M = T, a.N = R, a.K = dim, a.batch = H, a.exact = f32;
             if (int rc = vmx_linear_launch(a, st)) return rc;
         } else {
-            hipLaunchKernelGGL(zero_f32_kernel, dim3(1024), dim3(256), 0, st, m->qabs.as<float>(), (int64_t)T * H * R);
-            VMX_CHECK_LAUNCH("gesutar zero");
+            if (int rc = vmx_zero_f32(m->qabs.as<float>(), (int64_t)T * H * R, st)) return rc;
         }
         if (int rc = vmx_latent_attention(m->olat.as<float>(), m->qabs.as<float>(), m->qrot.as<float>(), L.cache.p, cdt, block_tables,
                                           max_blocks_per_seq, seq_ids, positions, L.sink.as<uint16_t>(), lc.scale, lc.window, T, H, R, rd,
@@ -533,9 +398,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         // ---- feed-forward: mixture of experts
         if (lc.mlp == VMX_MLP_MOE) {
             const int E = lc.experts, k = lc.top, ff = lc.expert_ff, pairs = T * k;
-            hipLaunchKernelGGL(rms_norm_f32in_kernel, dim3(T), dim3(256), 0, st, m->h.p, f32, x, (const int32_t *)nullptr, L.norm2.as<uint16_t>(),
-                               W, c.norm_eps);
-            VMX_CHECK_LAUNCH("gesutar norm2");
+            if (int rc = vmx_rms_norm_f32in(m->h.p, f32, x, nullptr, L.norm2.as<uint16_t>(), 0, W, c.norm_eps, T, st)) return rc;
             VmxLinear r;   // router logits: always a true f32 product
             r.A = m->h.p, r.a_f32 = f32, r.lda = W;
             r.W = L.router.as<uint16_t>(), r.w_sn = W, r.w_sk = 1;
@@ -547,21 +410,19 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
             if (int rc = vmx_grouped_topk_router(m->rlogits.as<float>(), m->topw.as<float>(), m->topi.as<int32_t>(), T, E, k, lc.groups,
                                                  lc.keep_groups, lc.router_scale, st))
                 return rc;
-            const bool few = pairs <= FEW_PAIRS;   // every pair its own block: no sort, an expert's weights are read once per pair
+            const bool few = pairs <= VMX_MOE_FEW_PAIRS;   // every pair its own block: no sort, an expert's weights are read once per pair
             const int br = few ? 16 : (pairs >= 32 * E ? 64 : 16);
             const int cap = few ? pairs * 16 : pairs + E * (br - 1);
             const int32_t *fp = m->few_pairs.as<int32_t>();
-            const int32_t *up_rows = few ? fp : m->sorted.as<int32_t>(), *down_rows = few ? fp + FEW_PAIRS * 16 : nullptr;
+            const int32_t *up_rows = few ? fp : m->sorted.as<int32_t>(), *down_rows = few ? fp + VMX_MOE_FEW_PAIRS * 16 : nullptr;
             const int32_t *blk = few ? m->topi.as<int32_t>() : m->blk_expert.as<int32_t>();
-            const int32_t *total = few ? fp + 2 * FEW_PAIRS * 16 + FEW_PAIRS : m->total.as<int32_t>();
-            const int32_t *inv = few ? fp + 2 * FEW_PAIRS * 16 : m->inv.as<int32_t>();
+            const int32_t *total = few ? fp + 2 * VMX_MOE_FEW_PAIRS * 16 + VMX_MOE_FEW_PAIRS : m->total.as<int32_t>();
+            const int32_t *inv = few ? fp + 2 * VMX_MOE_FEW_PAIRS * 16 : m->inv.as<int32_t>();
             if (!few) {
                 if (int rc = vmx_moe_align_block_size(m->topi.as<int32_t>(), m->sorted.as<int32_t>(), m->blk_expert.as<int32_t>(),
                                                       m->total.as<int32_t>(), pairs, E, br, cap, st))
                     return rc;
-                hipLaunchKernelGGL(moe_inverse_kernel, dim3((cap + 255) / 256), dim3(256), 0, st, m->inv.as<int32_t>(), m->sorted.as<int32_t>(),
-                                   m->total.as<int32_t>(), pairs);
-                VMX_CHECK_LAUNCH("gesutar moe inverse");
+                if (int rc = vmx_moe_inverse(m->inv.as<int32_t>(), m->sorted.as<int32_t>(), m->total.as<int32_t>(), pairs, cap, st)) return rc;
             }
             VmxLinear u;   // act = relu(W_up[e] h)^2 over the pairs' rows
             u.A = m->h.p, u.a_f32 = f32, u.lda = W;
@@ -595,16 +456,13 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
                 if (int rc = vmx_linear_launch(sd, st)) return rc;
                 shared = m->sout.as<float>();
             }
-            hipLaunchKernelGGL(moe_combine_f32_kernel, dim3((W + 255) / 256, T), dim3(256), 0, st, x, m->ydown.as<float>(), inv, m->topw.as<float>(), k, shared, W);
-            VMX_CHECK_LAUNCH("gesutar moe combine");
+            if (int rc = vmx_moe_combine_f32(x, m->ydown.as<float>(), inv, m->topw.as<float>(), k, shared, nullptr, 0, T, W, st)) return rc;
         }
         if (layer_trace)
             VMX_CHECK_HIP(hipMemcpyAsync(layer_trace + (size_t)li * T * W, x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
     }
     if (num_logit_rows > 0) {
-        hipLaunchKernelGGL(rms_norm_f32in_kernel, dim3(num_logit_rows), dim3(256), 0, st, m->hsel.p, f32, x, logit_rows,
-                           m->final_norm.as<uint16_t>(), W, c.norm_eps);
-        VMX_CHECK_LAUNCH("gesutar final norm");
+        if (int rc = vmx_rms_norm_f32in(m->hsel.p, f32, x, logit_rows, m->final_norm.as<uint16_t>(), 0, W, c.norm_eps, num_logit_rows, st)) return rc;
         float *lg = logits ? logits : m->fused.as<float>();   // greedy ids only: the logits live in a workspace
         VMX_REQUIRE(logits || (size_t)num_logit_rows * c.vocab * 4 <= m->fused.bytes, "gesutar_forward: pass a logits buffer for %d rows",
                     num_logit_rows);
@@ -615,11 +473,7 @@ extern "C" int vmx_gesutar_forward(vmx_gesutar *m, const int32_t *tokens, const 
         hd.M = num_logit_rows, hd.N = c.vocab, hd.K = W, hd.exact = f32;
         if (int rc = vmx_linear_launch(hd, st)) return rc;
         if (greedy_ids) {
-            const int chunks = (c.vocab + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
-            hipLaunchKernelGGL(argmax_f32_partial_kernel, dim3(chunks, num_logit_rows), dim3(256), 0, st, m->argmax_keys.as<unsigned long long>(), lg,
-                               c.vocab, chunks);
-            hipLaunchKernelGGL(argmax_f32_final_kernel, dim3(num_logit_rows), dim3(64), 0, st, greedy_ids, m->argmax_keys.as<unsigned long long>(), chunks);
-            VMX_CHECK_LAUNCH("gesutar argmax");
+            if (int rc = vmx_argmax_f32_rows(greedy_ids, m->argmax_keys.as<unsigned long long>(), lg, num_logit_rows, c.vocab, st)) return rc;
         }
     }
     return VMX_OK;

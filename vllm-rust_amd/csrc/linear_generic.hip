@@ -5,7 +5,8 @@
 //   * blockIdx.z batches with element strides (one product per attention head);
 //   * gathered activation rows and per-row-block weight matrices (experts of a mixture whose (token, slot) pairs were sorted into
 //     blocks by vmx_moe_align_block_size);
-//   * epilogues: plain store, squared ReLU, accumulate into an f32 residual stream, multiply by sigmoid(gate).
+//   * an optional bf16 bias per output column, then an epilogue: plain store, squared ReLU, tanh-form GELU, accumulate into an
+//     f32 residual stream, multiply by sigmoid(gate), or both of the last two (a gated residual update).
 // Kernels: `linear_mfma_kernel` (64-row tiles for prompts and 64-row expert blocks; a staged 16-row form for shapes the streaming
 // kernel does not take) and `linear_skinny_kernel` (up to 16 rows: decode steps and 16-row expert blocks, weights streamed once)
 // round the activations to bf16 and run v_mfma_f32_16x16x32_bf16; `linear_fma_kernel` multiplies in true f32 on the vector ALU
@@ -21,15 +22,18 @@ __device__ __forceinline__ float ld_act(const void *A, int a_f32, int64_t i) {
 }
 
 __device__ __forceinline__ void linear_store(const VmxLinear &p, int z, int m, int n, float v) {
+    if (p.bias) v += vmx_bf16_to_f32(p.bias[n + z * p.bias_bs]);
     if (p.epilogue == VMX_EP_RELU2) {
         const float r = fmaxf(v, 0.f);
         v = r * r;
-    } else if (p.epilogue == VMX_EP_MUL_SIGMOID) {
+    } else if (p.epilogue == VMX_EP_GELU_TANH) {
+        v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    } else if (p.epilogue == VMX_EP_MUL_SIGMOID || p.epilogue == VMX_EP_ADD_MUL_SIGMOID) {
         const float g = p.aux[(int64_t)m * p.ldaux + n + z * p.aux_bs];
         v *= 1.0f / (1.0f + expf(-g));
     }
     const int64_t o = (int64_t)m * p.ldc + n + z * p.c_bs;
-    if (p.epilogue == VMX_EP_ADD_F32) ((float *)p.C)[o] += v;
+    if (p.epilogue == VMX_EP_ADD_F32 || p.epilogue == VMX_EP_ADD_MUL_SIGMOID) ((float *)p.C)[o] += v;
     else if (p.c_f32) ((float *)p.C)[o] = v;
     else ((uint16_t *)p.C)[o] = vmx_f32_to_bf16(v);
 }
@@ -340,8 +344,8 @@ __global__ __launch_bounds__(256) void linear_fewcols_f32_kernel(const VmxLinear
 int vmx_linear_launch(const VmxLinear &p, hipStream_t st) {
     VMX_REQUIRE(p.A && p.W && p.C, "linear: null pointer");
     VMX_REQUIRE(p.M >= 0 && p.N > 0 && p.K > 0 && p.batch >= 1, "linear: bad shape M %d N %d K %d batch %d", p.M, p.N, p.K, p.batch);
-    VMX_REQUIRE(p.epilogue != VMX_EP_ADD_F32 || p.c_f32, "linear: the accumulating epilogue needs an f32 output");
-    VMX_REQUIRE(p.epilogue != VMX_EP_MUL_SIGMOID || p.aux, "linear: the gate epilogue needs its gate rows");
+    VMX_REQUIRE((p.epilogue != VMX_EP_ADD_F32 && p.epilogue != VMX_EP_ADD_MUL_SIGMOID) || p.c_f32, "linear: the accumulating epilogues need an f32 output");
+    VMX_REQUIRE((p.epilogue != VMX_EP_MUL_SIGMOID && p.epilogue != VMX_EP_ADD_MUL_SIGMOID) || p.aux, "linear: the gate epilogues need their gate rows");
     VMX_REQUIRE(!p.block_expert || (p.total_rows && (p.block_rows == 16 || p.block_rows == 64)), "linear: expert blocks are 16 or 64 rows");
     VMX_REQUIRE(!p.row_ids || p.row_div >= 1, "linear: row_div must be positive");
     if (p.M == 0) return VMX_OK;

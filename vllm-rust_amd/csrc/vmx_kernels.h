@@ -174,7 +174,7 @@ bool vmx_q3k_gemm16_ok(int n_out, int n_in, int m);
 int vmx_q3k_gemm16_bf16(const void *w, const uint16_t *x, float *y, int n_out, int n_in, int m, hipStream_t st);
 
 // linear_generic.hip: linear layers over unquantized bf16 weights of any shape (f32 accumulation in ascending k)
-enum { VMX_EP_STORE = 0, VMX_EP_RELU2 = 1, VMX_EP_ADD_F32 = 2, VMX_EP_MUL_SIGMOID = 3 };
+enum { VMX_EP_STORE = 0, VMX_EP_RELU2 = 1, VMX_EP_ADD_F32 = 2, VMX_EP_MUL_SIGMOID = 3, VMX_EP_GELU_TANH = 4, VMX_EP_ADD_MUL_SIGMOID = 5 };
 struct VmxLinear {
     const void *A = nullptr;           // activations [M, K], K contiguous, rows lda elements apart
     int a_f32 = 0;                     // 1: f32 activations, 0: bf16
@@ -193,9 +193,50 @@ struct VmxLinear {
     int64_t expert_stride = 0;
     int block_rows = 0;
     const int32_t *total_rows = nullptr;     // device scalar: row blocks at or past it do nothing
-    int epilogue = VMX_EP_STORE;       // RELU2: max(v, 0)^2; ADD_F32: C += v (f32 C); MUL_SIGMOID: v * sigmoid(aux[m, n])
+    const uint16_t *bias = nullptr;    // bf16 [N] added to the sum before the epilogue (batches bias_bs elements apart)
+    int64_t bias_bs = 0;
+    int epilogue = VMX_EP_STORE;       // RELU2: max(v, 0)^2; GELU_TANH; ADD_F32: C += v (f32 C); MUL_SIGMOID: v * sigmoid(aux[m, n]);
+                                       // ADD_MUL_SIGMOID: C += v * sigmoid(aux[m, n]) (f32 C)
     const float *aux = nullptr;
     int64_t ldaux = 0;
     int exact = 0;                     // 1: multiply in f32 on the vector ALU even where the matrix cores could take bf16 operands
 };
 int vmx_linear_launch(const VmxLinear &p, hipStream_t st);
+
+// packed_ops.hip: what the packed-step executors share
+// A device allocation owned by an executor (host-side handle).
+struct VmxBuf {
+    void *p = nullptr;
+    size_t bytes = 0;
+    int alloc(size_t n) {
+        release();
+        bytes = n;
+        hipError_t e = hipMalloc(&p, n ? n : 16);
+        if (e != hipSuccess) {
+            p = nullptr;
+            vmx_set_error("hipMalloc(%zu) failed: %s", n, hipGetErrorString(e));
+            return VMX_ENOMEM;
+        }
+        return VMX_OK;
+    }
+    void release() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+    }
+    template <typename T> T *as() const { return (T *)p; }
+};
+constexpr int VMX_ARGMAX_CHUNK = 1024;     // logits per workgroup of the first argmax pass: keys [rows][ceil(vocab / chunk)]
+constexpr int VMX_MOE_FEW_PAIRS = 16;      // most (token, slot) pairs of a step that runs its experts unsorted, one 16-row block per pair
+// out[r] = x[rows ? rows[r] : r] / sqrt(mean(x^2) + eps) * w (w_scalar: w[0] for every column); out f32 or bf16 [n, width]
+int vmx_rms_norm_f32in(void *out, int out_f32, const float *x, const int32_t *rows, const uint16_t *w, int w_scalar, int width, float eps,
+                       int n, hipStream_t st);
+int vmx_zero_f32(float *p, int64_t n, hipStream_t st);
+// inv[pair] = place of the pair in the expert-sorted list (vmx_moe_align_block_size)
+int vmx_moe_inverse(int32_t *inv, const int32_t *sorted, const int32_t *total, int numel, int cap, hipStream_t st);
+// x[t] += (sum_slot w[t, slot] * y[inv[t k + slot]] + shared[t]) * sigmoid(gate[t * ldgate ..]); shared and gate may be NULL
+int vmx_moe_combine_f32(float *x, const float *y, const int32_t *inv, const float *w, int k, const float *shared, const float *gate,
+                        int64_t ldgate, int T, int width, hipStream_t st);
+int vmx_argmax_f32_rows(int32_t *out, unsigned long long *keys, const float *logits, int rows, int vocab, hipStream_t st);
+int vmx_embed_scaled_f32(float *x, const uint16_t *embed, const int32_t *tokens, int T, int width, int vocab, float scale, hipStream_t st);
+// act[r, j] = silu(gu[r, j]) * gu[r, ff + j], gu f32 [rows, 2 ff], act f32 or bf16 [rows, ff]
+int vmx_glu_silu_rows(void *act, int act_f32, const float *gu, int rows, int ff, hipStream_t st);

@@ -41,14 +41,33 @@ class BlockManager:
         self.free.extend(blocks)
 
 
+class StateSlots:
+    """Free list of recurrent-state slots: a model with recurrent layers keeps each live sequence's state (convolution inputs,
+    matrix memories) in one slot of fixed size.  A slot is not cleared when it changes hands: the executor starts a sequence whose
+    step begins at position 0 from zeros.  Like the blocks, freed slots are handed out again first."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free = list(range(num_slots - 1, -1, -1))
+
+    def allocate(self) -> int:
+        if not self.free:
+            raise MemoryError(f"all {self.num_slots} state slots are in use")
+        return self.free.pop()
+
+    def release(self, slot: int) -> None:
+        self.free.append(slot)
+
+
 @dataclasses.dataclass
 class Sequence:
-    """What a request holds between steps: its cache blocks, how many tokens they hold, and its last token (the hashed bigram
-    embedding of the next token needs it)."""
+    """What a request holds between steps: its cache blocks, how many tokens they hold, its last token (the hashed bigram
+    embedding of the next token needs it) and, for models with recurrent layers, its state slot."""
     seq_id: object
     blocks: list = dataclasses.field(default_factory=list)
     length: int = 0
     last_token: int = -1
+    state_slot: int = -1
 
 
 @dataclasses.dataclass
@@ -63,9 +82,11 @@ class SamplingParams:
 class Engine:
     def __init__(self, model, max_tokens: int | None = None):
         """model: an executor driver with .forward(tokens, prev, positions, slots, seq_ids, block_tables, logit_rows, ...),
-        .block_size, .num_blocks, .max_tokens, .vocab_size (GesutarForCausalLM; PackedQwen3 adapts the Qwen3 executor)."""
+        .block_size, .num_blocks, .max_tokens, .vocab_size (GesutarForCausalLM, GupuvikForCausalLM; PackedQwen3 adapts the Qwen3
+        executor).  A driver with .state_slots > 0 also gets seq_starts and state_slots (recurrent state per sequence)."""
         self.model = model
         self.blocks = BlockManager(model.num_blocks, model.block_size)
+        self.states = StateSlots(model.state_slots) if getattr(model, "state_slots", 0) else None
         self.max_tokens = min(max_tokens or model.max_tokens, model.max_tokens)
         self.seqs: dict = {}
         self.device = model.device
@@ -74,13 +95,19 @@ class Engine:
     def add(self, seq_id) -> Sequence:
         if seq_id in self.seqs:
             raise KeyError(f"sequence {seq_id!r} already exists")
-        s = self.seqs[seq_id] = Sequence(seq_id)
+        s = Sequence(seq_id)
+        if self.states is not None:
+            s.state_slot = self.states.allocate()
+        self.seqs[seq_id] = s
         return s
 
     def finish(self, seq_id) -> None:
         s = self.seqs.pop(seq_id)
         self.blocks.release(s.blocks)
         s.blocks = []
+        if self.states is not None and s.state_slot >= 0:
+            self.states.release(s.state_slot)
+            s.state_slot = -1
 
     def _dev(self, a) -> torch.Tensor:
         return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(self.device)
@@ -126,8 +153,14 @@ class Engine:
         bt = np.zeros((len(seqs), width), np.int32)
         for i, s in enumerate(seqs):
             bt[i, :len(s.blocks)] = s.blocks
+        extra = {}
+        if self.states is not None:   # recurrent layers walk each sequence's rows in order and carry its state slot
+            starts = np.zeros(len(seqs) + 1, np.int32)
+            starts[1:] = np.cumsum([len(t) for _, t, _ in entries])
+            extra = {"seq_starts": self._dev(starts), "state_slots": self._dev([s.state_slot for s in seqs])}
         out = self.model.forward(self._dev(tok), self._dev(prev), self._dev(pos), self._dev(slots), self._dev(sid), self._dev(bt),
-                                 self._dev(rows) if rows else None, want_logits=want_logits, want_greedy=want_greedy, layer_trace=layer_trace)
+                                 self._dev(rows) if rows else None, want_logits=want_logits, want_greedy=want_greedy, layer_trace=layer_trace,
+                                 **extra)
         for s, (_, tokens, _) in zip(seqs, entries):
             s.length += len(tokens)
             s.last_token = int(tokens[-1])
