@@ -384,7 +384,7 @@ extern "C" int vmx_gupuvik_forward(vmx_gupuvik *m, const int32_t *tokens, const 
             Layer &S = lc.kv_from < 0 ? L : m->layers[lc.kv_from];
             if (int rc = vmx_window_attention(m->attn.p, cdt, fused + L.q_off, nf, S.kcache.p, S.vcache.p, cdt, block_tables, max_blocks_per_seq,
                                               seq_ids, positions, L.temp.as<uint16_t>(), fused + L.g_off, nf, lc.scale, lc.softcap, lc.window,
-                                              lc.keep_first, T, H, G, D, V, c.block_size, st))
+                                              lc.keep_first, T, H, G, D, V, c.block_size, seq_starts, num_seqs, st))
                 return rc;
         } else {
             const int C = 2 * G * D + H * V;

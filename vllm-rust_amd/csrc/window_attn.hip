@@ -8,8 +8,9 @@
 // Keys and values live in two caches of rows [kv_heads * dim] / [kv_heads * vdim], bf16 or f32; a step writes its new rows first
 // (vmx_kv_cache_write_f32) and prompts, prompt portions and decode tokens then run the SAME kernel over the cache, so a row's
 // result does not depend on how its prompt was cut or on what else is in the step.  Scores, softmax and the weighted sum are f32.
-// The visible keys of a row are two runs, [0, min(keep_first, lo)) and [lo, i] with lo = max(0, i - window + 1); a wave owns one
-// (token, head) row and walks them 64 at a time: lane l scores key l of the tile, then every lane sums its value columns.
+// The visible keys of a row are two runs, [0, min(keep_first, lo)) and [lo, i] with lo = max(0, i - window + 1).  Two kernels:
+// the vector form (any sizes, f32 or bf16 cache: a wave owns one (token, head) row and walks its keys 64 at a time, lane l scores
+// key l of the tile, then every lane sums its value columns) and the matrix-core form below for bf16 caches.
 #include "vmx_kernels.h"
 #include <float.h>
 
@@ -51,6 +52,8 @@ struct WinAttn {
     int64_t ldgate;
     float scale, softcap;
     int window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size;
+    const int32_t *seq_starts;   // matrix-core form: sequence s owns the packed rows seq_starts[s] .. seq_starts[s + 1] - 1
+    int num_seqs;
 };
 
 constexpr int WA_MAX_DIM = 256;
@@ -120,6 +123,193 @@ __global__ __launch_bounds__(256) void window_attn_wave_kernel(const WinAttn p) 
     }
 }
 
+// Matrix-core form over a bf16 cache (dim and vdim multiples of 8, dim <= 32 DS, vdim <= 16 VS).  A workgroup owns one key/value
+// head and a run of up to 16 nt consecutive rows of ONE sequence (found from seq_starts, so decode batches and unequal prompts
+// need no padding); wave w owns 16 of these rows for one of the query heads that share the key/value head (nt = 4 / heads per
+// key/value head, at most 4 heads per pass, the rest on blockIdx.z).  The run's visible keys, [0, min(keep, lo)) and [lo, last
+// row], are walked in tiles of 64: key rows are staged row-major in LDS (one tile ahead, through registers), value rows
+// transposed, with the keys of a tile permuted so that the scores a lane holds are the k slots of its next operand:
+//   S^T = K Q^T   (A = key rows from LDS, B = the wave's query fragments, kept in registers): lane (c, g) gets the scores of
+//                 query c against keys 16 kt + 4 g + r;
+//   O^T += V^T P^T (A = transposed value rows from LDS, B = those scores after the softmax, as a bf16 pair hi + lo so that the
+//                 weights keep f32 precision): lane (c, g) accumulates value columns 16 vs + 4 g + r of query c.
+// Every statistic of a query therefore lives in the four lanes (c, 0..3): the softmax needs two lane exchanges per tile.
+template <int DS, int VS>
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) {
+    constexpr int KT = 64, LDK = 32 * DS + 8, LDV = KT + 8, KCH = DS, VCH = (VS + 1) / 2;
+    __shared__ __align__(16) uint16_t Ks[KT * LDK];
+    __shared__ __align__(16) uint16_t Vt[16 * VS * LDV];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
+    const int qpk = p.heads / p.kv_heads, hq = min(qpk, 4), nt = 4 / hq, RT = 16 * nt;
+    int tile = blockIdx.x, r0 = 0, nrows = 0;
+    for (int s = 0; s < p.num_seqs; s++) {
+        const int a = p.seq_starts[s], len = p.seq_starts[s + 1] - a, n = (len + RT - 1) / RT;
+        if (tile < n) {
+            r0 = a + tile * RT;
+            nrows = min(RT, len - tile * RT);
+            break;
+        }
+        tile -= n;
+    }
+    if (nrows <= 0) return;   // the same for the whole workgroup
+    const int kvh = blockIdx.y, sub = wave / hq, hh = blockIdx.z * 4 + wave % hq;
+    const bool active = sub < nt && hh < qpk && 16 * sub < nrows;
+    const int head = kvh * qpk + (hh < qpk ? hh : 0);
+    const int D = p.dim, V = p.vdim;
+    const int64_t kw = (int64_t)p.kv_heads * D, vw = (int64_t)p.kv_heads * V;
+    const int i0 = p.positions[r0], i1 = i0 + nrows - 1;
+    const int lo = p.window > 0 ? max(0, i0 - p.window + 1) : 0;
+    const int na = min(p.keep_first, lo), nk = na + (i1 - lo + 1);
+    const int32_t *bt = p.block_tables + (int64_t)p.seq_ids[r0] * p.max_blocks;
+    const uint16_t *kc = (const uint16_t *)p.kc, *vc = (const uint16_t *)p.vc;
+    const int qrow = 16 * sub + fl, qi = i0 + qrow;
+    const bool qlive = active && qrow < nrows;
+    uint4 qf[DS];
+#pragma unroll
+    for (int s = 0; s < DS; s++) {
+        const int k = 32 * s + 8 * fg;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (qlive && k < D) {
+            const float *src = p.q + (int64_t)(r0 + qrow) * p.ldq + (int64_t)head * D + k;
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = src[e];
+            v = vmx_pack16x8<false>(f);
+        }
+        qf[s] = v;
+    }
+    const float smul = p.scale * (p.temp ? vmx_bf16_to_f32(p.temp[head]) : 1.0f);
+    const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
+    uint4 kr[KCH], vr[VCH];
+    auto cache_row = [&](int idx) -> int64_t {
+        const int j = idx < na ? idx : lo + (idx - na);
+        return (int64_t)bt[j / p.block_size] * p.block_size + j % p.block_size;
+    };
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int c = 0; c < KCH; c++) {
+            const int ch = tid + 256 * c, kk = ch / (4 * DS), part = ch % (4 * DS);
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (kb + kk < nk && 8 * part < D) v = *reinterpret_cast<const uint4 *>(kc + cache_row(kb + kk) * kw + (int64_t)kvh * D + 8 * part);
+            kr[c] = v;
+        }
+#pragma unroll
+        for (int c = 0; c < VCH; c++) {
+            const int ch = tid + 256 * c, kk = ch / (2 * VS), part = ch % (2 * VS);
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (ch < KT * 2 * VS && kb + kk < nk && 8 * part < V) v = *reinterpret_cast<const uint4 *>(vc + cache_row(kb + kk) * vw + (int64_t)kvh * V + 8 * part);
+            vr[c] = v;
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int c = 0; c < KCH; c++) {
+            const int ch = tid + 256 * c, kk = ch / (4 * DS), part = ch % (4 * DS);
+            *reinterpret_cast<uint4 *>(Ks + kk * LDK + 8 * part) = kr[c];
+        }
+#pragma unroll
+        for (int c = 0; c < VCH; c++) {
+            const int ch = tid + 256 * c, kk = ch / (2 * VS), part = ch % (2 * VS);
+            if (ch < KT * 2 * VS) {
+                // key kk of the tile sits in k slot `col`: the order in which the score registers of a lane line up as an operand
+                const int col = 32 * (kk >> 5) + 8 * ((kk & 15) >> 2) + (kk & 3) + 4 * ((kk >> 4) & 1);
+                const uint32_t w[4] = {vr[c].x, vr[c].y, vr[c].z, vr[c].w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) Vt[(8 * part + e) * LDV + col] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    };
+    float m = -FLT_MAX, den = 0.f;
+    vmx_f32x4 o[VS];
+#pragma unroll
+    for (int v = 0; v < VS; v++) o[v] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
+    fetch(0);
+    stash();
+    __syncthreads();
+    for (int kb = 0; kb < nk; kb += KT) {
+        if (kb + KT < nk) fetch(kb + KT);
+        if (active) {
+            float sc[4][4];
+            float tmax = -FLT_MAX;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++) {
+                vmx_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < DS; s++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(Ks + (16 * kt + fl) * LDK + 32 * s + 8 * fg);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, a), __builtin_bit_cast(vmx_bf16x8, qf[s]), acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int idx = kb + 16 * kt + 4 * fg + r;
+                    const int j = idx < na ? idx : lo + (idx - na);
+                    const bool vis = qlive && idx < nk && j <= qi && (p.window == 0 || qi - j < p.window || j < p.keep_first);
+                    float x = acc[r] * smul;
+                    if (p.softcap > 0.f) x = p.softcap * tanhf(x * inv_cap);
+                    sc[kt][r] = vis ? x : -FLT_MAX;
+                    tmax = fmaxf(tmax, sc[kt][r]);
+                }
+            }
+            tmax = fmaxf(tmax, vmx_lane_xor<16>(tmax));
+            tmax = fmaxf(tmax, vmx_lane_xor<32>(tmax));
+            const float mn = fmaxf(m, tmax);
+            const float f = expf(m - mn);
+            float psum = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    sc[kt][r] = sc[kt][r] > -FLT_MAX ? expf(sc[kt][r] - mn) : 0.f;
+                    psum += sc[kt][r];
+                }
+            psum += vmx_lane_xor<16>(psum);
+            psum += vmx_lane_xor<32>(psum);
+            den = den * f + psum;
+            m = mn;
+#pragma unroll
+            for (int v = 0; v < VS; v++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[v][r] *= f;
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                float hi[8], lw[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float pv = sc[2 * u + (e >> 2)][e & 3];
+                    hi[e] = vmx_bf16_to_f32(vmx_f32_to_bf16(pv));
+                    lw[e] = pv - hi[e];
+                }
+                const uint4 bh = vmx_pack16x8<false>(hi), bl = vmx_pack16x8<false>(lw);
+#pragma unroll
+                for (int v = 0; v < VS; v++) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(Vt + (16 * v + fl) * LDV + 32 * u + 8 * fg);
+                    o[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, a), __builtin_bit_cast(vmx_bf16x8, bh), o[v], 0, 0, 0);
+                    o[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(vmx_bf16x8, a), __builtin_bit_cast(vmx_bf16x8, bl), o[v], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+        if (kb + KT < nk) {
+            stash();
+            __syncthreads();
+        }
+    }
+    if (!qlive) return;
+    float g = 1.0f / den;
+    if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)(r0 + qrow) * p.ldgate + head]));
+#pragma unroll
+    for (int v = 0; v < VS; v++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int c = 16 * v + 4 * fg + r;
+            if (c < V) {
+                const int64_t at = ((int64_t)(r0 + qrow) * p.heads + head) * V + c;
+                if (p.out_f32) ((float *)p.out)[at] = o[v][r] * g;
+                else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(o[v][r] * g);
+            }
+        }
+}
+
 }  // namespace
 
 extern "C" int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *v, int64_t ldv, const int32_t *slots, void *k_cache,
@@ -138,7 +328,7 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
                                     int cache_dtype, const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids,
                                     const int32_t *positions, const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale,
                                     float softcap, int window, int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim,
-                                    int block_size, void *stream) {
+                                    int block_size, const int32_t *seq_starts, int num_seqs, void *stream) {
     VMX_REQUIRE(out && q && k_cache && v_cache && block_tables && seq_ids && positions, "window_attention: null pointer");
     VMX_REQUIRE((out_dtype == VMX_F32 || out_dtype == VMX_BF16) && (cache_dtype == VMX_F32 || cache_dtype == VMX_BF16),
                 "window_attention: f32 or bf16 output and cache");
@@ -149,10 +339,33 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
     VMX_REQUIRE(ldq >= (int64_t)heads * dim && (!gate || ldgate >= heads), "window_attention: bad row strides");
     if (tokens <= 0) return VMX_OK;
     WinAttn p{out, out_dtype == VMX_F32, q, ldq, k_cache, v_cache, block_tables, seq_ids, positions, max_blocks_per_seq, head_temp_bf16,
-              gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size};
-    const dim3 grid((tokens * heads + 3) / 4), block(256);
+              gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size, seq_starts, num_seqs};
     hipStream_t st = vmx_stream(stream);
     const bool f32 = cache_dtype == VMX_F32;
+    if (!f32 && seq_starts && num_seqs >= 1 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 128 && ldq % 4 == 0 && ((uintptr_t)q & 15) == 0 &&
+        ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0) {
+        const int qpk = heads / kv_heads, hq = qpk < 4 ? qpk : 4, rt = 16 * (4 / hq);
+        const dim3 mgrid(tokens / rt + num_seqs, kv_heads, (qpk + 3) / 4);   // at most one partly filled run per sequence
+        const int ds = dim <= 64 ? 2 : (dim <= 128 ? 4 : 8), vs = vdim <= 32 ? 2 : (vdim <= 64 ? 4 : 8);
+#define WM_LAUNCH(A, B) hipLaunchKernelGGL((window_attn_mfma_kernel<A, B>), mgrid, dim3(256), 0, st, p)
+        if (ds == 2) {
+            if (vs == 2) WM_LAUNCH(2, 2);
+            else if (vs == 4) WM_LAUNCH(2, 4);
+            else WM_LAUNCH(2, 8);
+        } else if (ds == 4) {
+            if (vs == 2) WM_LAUNCH(4, 2);
+            else if (vs == 4) WM_LAUNCH(4, 4);
+            else WM_LAUNCH(4, 8);
+        } else {
+            if (vs == 2) WM_LAUNCH(8, 2);
+            else if (vs == 4) WM_LAUNCH(8, 4);
+            else WM_LAUNCH(8, 8);
+        }
+#undef WM_LAUNCH
+        VMX_CHECK_LAUNCH("window_attention (matrix cores)");
+        return VMX_OK;
+    }
+    const dim3 grid((tokens * heads + 3) / 4), block(256);
     const int vpl = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
 #define WA_LAUNCH(F, U) hipLaunchKernelGGL((window_attn_wave_kernel<F, U>), grid, block, 0, st, p)
     if (f32) {

@@ -83,8 +83,11 @@ class GupuvikLayerSpec:
 
     def to_config(self) -> dict:
         if self.mixer == "attention":
-            m = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
-                 "softcap": self.softcap, "mask": {"size": self.window, "keep_first": self.keep_first}}
+            m = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+            if self.softcap:
+                m["softcap"] = self.softcap
+            if self.window:                  # no window: every earlier key is visible and there is no mask to state
+                m["mask"] = {"size": self.window, "keep_first": self.keep_first}
             if self.kv_from is not None:
                 m["kv_from"] = self.kv_from
         else:
