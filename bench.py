@@ -758,6 +758,112 @@ def gesutar_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16))
             "data": "synthetic", "prompt": prompt, "sizes": out}
 
 
+GUPUVIK_SIZES = {
+    # name: (width, heads, kv_heads, dim, vdim, window, keep_first, experts, top, expert_ff, conv, rank, vocab, Gesutar kv_rank, Gesutar rot_dim)
+    "1k": (1024, 8, 2, 128, 128, 1024, 4, 16, 4, 512, 4, 64, 32000, 256, 32),
+    "2k": (2048, 16, 4, 128, 128, 4096, 4, 32, 4, 1024, 4, 128, 32000, 512, 64),
+}
+
+
+def _packed_times(model, V, prompt, batches, warmup, steps, side, dev, recurrent):
+    """Prompt pass and decode steps of a packed-step executor (one hipGraph per step): {"prefill": s, B: s per step}."""
+    BM = max(batches)
+    per_seq = model.num_blocks // BM
+    i32 = lambda a: torch.as_tensor(a, dtype=torch.int32, device=dev).contiguous()   # noqa: E731
+    bt = torch.arange(per_seq * BM, dtype=torch.int32, device=dev).reshape(BM, per_seq).contiguous()
+    g = torch.Generator(device=dev).manual_seed(1)
+    toks = torch.randint(0, V, (prompt,), dtype=torch.int32, device=dev, generator=g)
+    prev = torch.cat([i32([-1]), toks[:-1]])
+    pos = torch.arange(prompt, dtype=torch.int32, device=dev)
+    last = i32([prompt - 1])
+    extra = lambda starts, slots: {"seq_starts": i32(starts), "state_slots": i32(slots)} if recurrent else {}   # noqa: E731
+    for b in range(BM):          # fill every sequence's cache and state (the first pass also pays the lazy set-up)
+        slots = (bt[b, (pos // 16).long()] * 16 + pos % 16).to(torch.int32)
+        sid = torch.zeros(prompt, dtype=torch.int32, device=dev)
+        model.forward(toks, prev, pos, slots, sid, bt[b:b + 1].contiguous(), last, want_logits=False, want_greedy=True, **extra([0, prompt], [b]))
+    torch.cuda.synchronize()
+    slots0 = (bt[0, (pos // 16).long()] * 16 + pos % 16).to(torch.int32)
+    sid0 = torch.zeros(prompt, dtype=torch.int32, device=dev)
+    ex0 = extra([0, prompt], [0])
+    out = {"prefill": _timed_graph(lambda: model.forward(toks, prev, pos, slots0, sid0, bt, last, want_logits=False, want_greedy=True, **ex0), side, 2, 10)}
+    for B in batches:
+        dtok = torch.randint(0, V, (B,), dtype=torch.int32, device=dev, generator=g)
+        dprev = torch.randint(0, V, (B,), dtype=torch.int32, device=dev, generator=g)
+        dpos = torch.full((B,), prompt, dtype=torch.int32, device=dev)
+        dslots = (bt[:B, prompt // 16] * 16 + prompt % 16).to(torch.int32).contiguous()
+        dsid = torch.arange(B, dtype=torch.int32, device=dev)
+        rows = torch.arange(B, dtype=torch.int32, device=dev)
+        exb = extra(list(range(B + 1)), list(range(B)))
+        out[B] = _timed_graph(lambda: model.forward(dtok, dprev, dpos, dslots, dsid, bt, rows, want_logits=False, want_greedy=True, **exb), side, warmup, steps)
+    return out
+
+
+def gupuvik_workload(prompt, steps, warmup, sizes=("1k", "2k"), batches=(1, 16)):
+    """Gupuvik (parallel gated-residual layers: window attention with kept first tokens / gated delta rule, dense and SiLU-gated
+    mixture feed-forwards, bf16 weights) at layer sizes of real models, beside the closest existing model at equal size: Gesutar,
+    the other packed-step executor over bf16 weights, with the same width, depth, head count, experts and vocabulary.  Four layers:
+    delta rule + dense, attention + experts, delta rule + experts, attention on the second layer's cache + experts.  Prompt pass:
+    tokens/s of one `prompt`-token sequence; decode: aggregate tok/s of B sequences at context `prompt`, one hipGraph per step."""
+    from vllm_rust_amd.gesutar import GesutarForCausalLM, GesutarLayerSpec, GesutarSpec
+    from vllm_rust_amd.gesutar import synthetic_weights as gesutar_weights
+    from vllm_rust_amd.gupuvik import GupuvikForCausalLM, GupuvikLayerSpec, GupuvikSpec, synthetic_weights
+    out = {}
+    dev = torch.device("cuda", torch.cuda.current_device())
+    side = torch.cuda.Stream(device=dev)
+    BM = max(batches)
+    per_seq = (prompt + warmup + steps + 8 + 15) // 16 + 1
+    for name in sizes:
+        W, H, G, dim, vd, win, keep, E, top, ff, conv, rank, V, R, rd = GUPUVIK_SIZES[name]
+        moe = dict(mlp="moe", experts=E, top=top, expert_ff=ff)
+        att = dict(mixer="attention", heads=H, kv_heads=G, dim=dim, vdim=vd, window=win, keep_first=keep, scale=1.0 / math.sqrt(dim), softcap=30.0)
+        dlt = dict(mixer="channel_delta", heads=H, kv_heads=H, dim=dim, vdim=vd, conv=conv, decay_rank=rank, gate_rank=rank)
+        layers = [GupuvikLayerSpec(**dlt, mlp="dense", ff=top * ff), GupuvikLayerSpec(**att, **moe), GupuvikLayerSpec(**dlt, **moe),
+                  GupuvikLayerSpec(**att, kv_from=1, **moe)]
+        spec = GupuvikSpec(vocab=V, width=W, layers=layers, embed_scale=1.0)
+        model = GupuvikForCausalLM(spec, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        model.load_state(synthetic_weights(spec, 3, device=dev))
+        t = _packed_times(model, V, prompt, batches, warmup, steps, side, dev, True)
+        model.close()
+        del model
+        NL = len(layers)
+        hv, hd = H * vd, H * dim
+        mix_att = W * (hd + 2 * G * dim + H) + hv * W          # q | k | v | head gates, output projection (the sharing layer has no k | v)
+        mix_dlt = W * (2 * hd + hv + H + 2 * rank) + rank * (hd + hv) + hv * W
+        gates = 2 * W * W
+        lin = 2 * mix_dlt + mix_att + (mix_att - W * 2 * G * dim) + NL * gates + 2 * W * top * ff + 3 * (top * 3 * ff + E) * W
+        att_fl = 2 * H * (dim + vd) * min(win, prompt / 2)      # two attention layers
+        dlt_fl = 2 * H * 3 * dim * vd                            # decay + two rank-one passes per token and head, two layers
+        res = {"prefill": {"tokens": prompt, "ms": round(t["prefill"] * 1e3, 3), "tok_s": round(prompt / t["prefill"], 1),
+                           "TFLOP_s": round(2.0 * prompt * (lin + att_fl + dlt_fl + V * W / prompt) / t["prefill"] / 1e12, 2)}}
+        wfixed = 2 * (2 * mix_dlt + mix_att + (mix_att - W * 2 * G * dim) + NL * gates + 2 * W * top * ff + 3 * E * W + V * W)
+        for B in batches:
+            by = wfixed + 2 * 3 * min(E, B * top) * 3 * ff * W + 2 * 2 * B * min(win + keep, prompt + 1) * G * (dim + vd) + 2 * 2 * B * H * dim * vd * 4
+            res[f"decode_b{B}"] = {"tok_s": round(B / t[B], 1), "ms_per_step": round(t[B] * 1e3, 4), "GBps_algorithmic": round(by / t[B] / 1e9, 1)}
+        # the closest existing model at equal size
+        gl = GesutarLayerSpec(heads=H, dim=dim - rd, rot_dim=rd, vdim=vd, kv_rank=R, window=win, rot_dims=rd, rot_base=1e6, scale=1.0 / math.sqrt(dim),
+                              experts=E, top=top, groups=4, keep_groups=2, expert_ff=ff, shared_ff=0, router_scale=1.0)
+        gs = GesutarSpec(vocab=V, width=W, layers=[gl] * NL, embed_scale=1.0, bigram_buckets=4093, bigram_mul_prev=31, bigram_mul_cur=7)
+        gm = GesutarForCausalLM(gs, "bfloat16", block_size=16, num_blocks=per_seq * BM, max_tokens=max(prompt, BM), max_seqs=BM)
+        gm.load_state(gesutar_weights(gs, 3, device=dev))
+        tg = _packed_times(gm, V, prompt, batches, warmup, steps, side, dev, False)
+        gm.close()
+        del gm
+        glin = NL * (W * (hd + R + rd + hv) + H * (dim - rd) * R + hv * R + hv * W + (top * 2 * ff + E) * W)
+        gres = {"prefill": {"tokens": prompt, "ms": round(tg["prefill"] * 1e3, 3), "tok_s": round(prompt / tg["prefill"], 1),
+                            "TFLOP_s": round(2.0 * prompt * (glin + NL * H * (2 * R + rd) * min(win, prompt / 2) + V * W / prompt) / tg["prefill"] / 1e12, 2)}}
+        gfixed = 2 * (NL * (W * (hd + R + rd + hv) + H * (dim - rd) * R + hv * R + hv * W + E * W) + V * W)
+        for B in batches:
+            by = gfixed + 2 * NL * min(E, B * top) * 2 * ff * W + 2 * NL * B * min(win, prompt + 1) * (R + rd)
+            gres[f"decode_b{B}"] = {"tok_s": round(B / tg[B], 1), "ms_per_step": round(tg[B] * 1e3, 4), "GBps_algorithmic": round(by / tg[B] / 1e9, 1)}
+        out[name] = {"gupuvik": res, "gesutar": gres,
+                     "config": {"width": W, "layers": ["channel_delta+dense", "attention+moe", "channel_delta+moe", "attention(kv of layer 1)+moe"],
+                                "heads": H, "kv_heads": G, "dim": dim, "vdim": vd, "window": win, "keep_first": keep, "experts": E, "top": top,
+                                "expert_ff": ff, "dense_ff": top * ff, "conv": conv, "rank": rank, "vocab": V,
+                                "gesutar": {"layers": NL, "kv_rank": R, "rot_dim": rd, "dim": dim - rd}}}
+    return {"metric": "Gupuvik prompt and decode throughput beside Gesutar at equal size", "unit": "tok/s", "dtype": "bf16", "data": "synthetic",
+            "prompt": prompt, "sizes": out}
+
+
 def plan_job(gpus, world, replicas_flag, weights, local_ranks):
     """What a launch of this script measures -- pure argument logic, no device.  N = 1: the single-GPU job.  N > 1 (one process
     per GPU under torch.distributed.run): ONE model tensor-parallel over the N ranks (BASELINE.json's metric is the TP curve at
@@ -914,11 +1020,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary measurements (other models at N = 1, replicas at N > 1)")
     ap.add_argument("--no-moe", action="store_true", help="skip the Mixtral-8x7B-shaped fused-MoE secondary measurement")
-    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar"], default="all",
+    ap.add_argument("--workload", choices=["all", "qwen3", "gemma4", "mixtral", "exl3", "gesutar", "gupuvik"], default="all",
                     help="profiling aid: run ONE workload alone (qwen3 = the primary without secondaries; the others print only "
                          "their own block), so that a kernel trace of the run holds that workload's launches only; gesutar = the Gesutar "
                          "executor (latent attention + grouped-router MoE, bf16) at two layer sizes beside the bf16 dense Qwen3 executor at "
-                         "equal size: prompt tok/s and decode tok/s at 1 and 16 sequences (not part of the default run)")
+                         "equal size: prompt tok/s and decode tok/s at 1 and 16 sequences (not part of the default run); gupuvik = the Gupuvik "
+                         "executor (window attention / gated delta rule, gated residuals, bf16) at two layer sizes beside Gesutar at equal size, "
+                         "the same measurements")
     ap.add_argument("--tp", action="store_true", help="accepted for compatibility: with --gpus N > 1 the tensor-parallel job is the default")
     ap.add_argument("--replicas", action="store_true",
                     help="with --gpus N > 1: N independent replicas as the primary (weak scaling, no collective) instead of ONE model "
@@ -933,8 +1041,10 @@ def main():
     plan = plan_job(args.gpus, world, args.replicas, args.weights, d.local)
 
     K_steps, W_steps = args.steps, args.warmup
-    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar"):   # one secondary alone (single GPU)
-        if args.workload == "gesutar":
+    if args.workload in ("gemma4", "mixtral", "exl3", "gesutar", "gupuvik"):   # one secondary alone (single GPU)
+        if args.workload == "gupuvik":
+            blk = gupuvik_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
+        elif args.workload == "gesutar":
             blk = gesutar_workload(max(args.prompt, 1024) if args.prompt == 256 else args.prompt, min(args.steps, 64), args.warmup)
         elif args.workload == "gemma4":
             blk = gemma4_secondary(args.prompt, max(16, K_steps // 2), W_steps, cpu_leg=not args.no_cpu_baseline)

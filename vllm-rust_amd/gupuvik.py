@@ -295,12 +295,17 @@ class GupuvikForCausalLM:
         if seq_starts is None or state_slots is None:
             raise ValueError("Gupuvik carries recurrent state: the step needs seq_starts and state_slots")
         T = tokens.numel()
+        S = seq_starts.numel() - 1           # the sequences of THIS step; the block table may hold more rows
+        if S < 1 or state_slots.numel() != S or block_tables.shape[0] < S:
+            raise ValueError(f"Gupuvik: {S} sequences by seq_starts, {state_slots.numel()} state slots, {block_tables.shape[0]} block-table rows")
+        if not all(a.numel() == T for a in (positions, slots, seq_ids)):
+            raise ValueError("Gupuvik: tokens, positions, slots and seq_ids must have one entry per token")
         n = 0 if logit_rows is None else logit_rows.numel()
         logits = torch.empty((n, self.spec.vocab), dtype=torch.float32, device=self.device) if n else None
         ids = torch.empty(n, dtype=torch.int32, device=self.device) if (n and want_greedy) else None
         trace = torch.empty((len(self.spec.layers), T, self.spec.width), dtype=torch.float32, device=self.device) if layer_trace else None
         check(lib.vmx_gupuvik_forward(self._h, tokens.data_ptr(), positions.data_ptr(), slots.data_ptr(), seq_ids.data_ptr(), T,
-                                      block_tables.data_ptr(), block_tables.shape[0], block_tables.shape[1], seq_starts.data_ptr(),
+                                      block_tables.data_ptr(), S, block_tables.shape[1], seq_starts.data_ptr(),
                                       state_slots.data_ptr(), None if not n else logit_rows.data_ptr(), n,
                                       None if logits is None else logits.data_ptr(), None if ids is None else ids.data_ptr(),
                                       None if trace is None else trace.data_ptr(), self._stream()))
