@@ -1032,12 +1032,15 @@ int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *v, int64_t 
  * the values, times sigmoid(gate[t * ldgate + h]) (NULL: none).  q f32 rows of heads * dim at stride ldq; out [tokens, heads * vdim]
  * f32 or bf16.  No rotation.  Scores and softmax in f32.  seq_starts [num_seqs + 1] (optional): sequence s owns the packed rows
  * seq_starts[s] .. seq_starts[s + 1] - 1 at consecutive positions; with it, a bf16 cache and sizes that are multiples of 8 (dim <= 256,
- * vdim <= 128) the products run on the matrix cores (queries as bf16, softmax weights as a bf16 pair), 16 rows of a sequence per wave. */
+ * vdim <= 128) the products run on the matrix cores (queries as bf16, softmax weights as a bf16 pair), 16 rows of a sequence per wave;
+ * launches of few rows then deal each run's keys to several workgroups and merge their sums, if a workspace is given
+ * (vmx_window_attention_workspace_bytes; NULL: no split). */
 int vmx_window_attention(void *out, int out_dtype, const float *q, int64_t ldq, const void *k_cache, const void *v_cache, int cache_dtype,
                          const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids, const int32_t *positions,
                          const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale, float softcap, int window,
                          int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim, int block_size, const int32_t *seq_starts,
-                         int num_seqs, void *stream);
+                         int num_seqs, void *workspace, size_t workspace_bytes, void *stream);
+size_t vmx_window_attention_workspace_bytes(int tokens, int heads, int vdim);
 
 /* Short causal convolution over time per channel with carried state, then SiLU: y[t, c] = silu(sum_s taps[c, n - 1 - s] x[t - s, c]);
  * inputs from before the step come from state[state_slots[seq]] ([taps - 1, channels] f32, the sequence's last inputs), inputs from

@@ -113,7 +113,8 @@ def feed(engine, seq_id, toks, cuts, finish=True):
 
 def _window_attention_op(torch, q, k, v, temp, gate, scale, cap, window, keep, block_size, dtype, seed=1, runs=False):
     """vmx_window_attention for ONE sequence whose blocks are scattered over a larger cache; every position is a query.
-    runs: tell the operator which rows form a sequence (it then takes its matrix-core form where the sizes and the cache allow)."""
+    runs: tell the operator which rows form a sequence (it then takes its matrix-core form where the sizes and the cache allow);
+    runs == "split": also hand it a workspace, so that it deals the keys of a run to several workgroups and merges."""
     from vllm_rust_amd._lib import check, lib
     T, H, D = q.shape
     G, V = k.shape[1], v.shape[2]
@@ -132,9 +133,11 @@ def _window_attention_op(torch, q, k, v, temp, gate, scale, cap, window, keep, b
     td = None if temp is None else temp.to(torch.bfloat16).cuda()
     gd = None if gate is None else gate.float().cuda()
     st = torch.tensor([0, T], dtype=torch.int32, device="cuda")
+    ws = torch.empty(lib.vmx_window_attention_workspace_bytes(T, H, V) // 4, dtype=torch.float32, device="cuda")
     check(lib.vmx_window_attention(out.data_ptr(), 0, qd.data_ptr(), H * D, kc.data_ptr(), vc.data_ptr(), dtype, bt.data_ptr(), nb, sid.data_ptr(),
                                    pid.data_ptr(), None if td is None else td.data_ptr(), None if gd is None else gd.data_ptr(), H, scale, cap, window,
-                                   keep, T, H, G, D, V, block_size, st.data_ptr() if runs else None, 1 if runs else 0, None))
+                                   keep, T, H, G, D, V, block_size, st.data_ptr() if runs else None, 1 if runs else 0,
+                                   ws.data_ptr() if runs == "split" else None, ws.numel() * 4, None))
     torch.cuda.synchronize()
     return out.cpu().double().view(T, H, V)
 
@@ -159,7 +162,7 @@ def _attention_want(torch, q, k, v, temp, gate, scale, cap, window, keep):
                                                        (6, 3, 33, 130, 5, 9, 2.0, 1), (1, 1, 64, 64, 1, 0, 0.0, 8), (2, 1, 8, 8, 3, 40, 5.0, 4),
                                                        (8, 2, 48, 32, 40, 7, 20.0, 16), (16, 2, 128, 128, 100, 0, 0.0, 16), (3, 3, 72, 24, 0, 0, 9.0, 2),
                                                        (6, 2, 136, 40, 20, 30, 0.0, 4)])
-@pytest.mark.parametrize("dtype,runs", [(0, False), (1, False), (1, True)])
+@pytest.mark.parametrize("dtype,runs", [(0, False), (1, False), (1, True), (1, "split")])
 def test_window_attention_operator(gpu, H, G, D, V, window, keep, cap, bs, dtype, runs):
     vmx, torch = gpu
     g = torch.Generator().manual_seed(H * 100 + D)
@@ -172,7 +175,7 @@ def test_window_attention_operator(gpu, H, G, D, V, window, keep, cap, bs, dtype
     assert float((got - want).abs().max()) <= 2e-5 * max(1.0, float(want.abs().max()))   # q holds bf16 values: both forms are exact in the operands
 
 
-@pytest.mark.parametrize("dtype,runs", [(0, False), (1, False), (1, True)])
+@pytest.mark.parametrize("dtype,runs", [(0, False), (1, False), (1, True), (1, "split")])
 @pytest.mark.parametrize("bs", [4, 16])
 def test_window_attention_needle_at_every_edge(gpu, dtype, runs, bs):
     """One key carries a score far above all others and a value nobody else has.  A query sees it exactly while it is inside the

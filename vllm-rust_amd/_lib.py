@@ -222,7 +222,8 @@ _SIGS = {
     "vmx_gesutar_missing_tensors": (_i, [_p]),
     "vmx_gesutar_forward": (_i, [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _p, _i, _p, _p, _p, _p]),
     "vmx_kv_cache_write_f32": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _p]),
-    "vmx_window_attention": (_i, [_p, _i, _p, _i64, _p, _p, _i, _p, _i, _p, _p, _p, _p, _i64, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p]),
+    "vmx_window_attention": (_i, [_p, _i, _p, _i64, _p, _p, _i, _p, _i, _p, _p, _p, _p, _i64, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _sz, _p]),
+    "vmx_window_attention_workspace_bytes": (_sz, [_i, _i, _i]),
     "vmx_short_conv_state_bytes": (_sz, [_i, _i, _i]),
     "vmx_short_conv_silu": (_i, [_p, _i64, _p, _p, _p, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p]),
     "vmx_short_conv_state_update": (_i, [_p, _i64, _p, _p, _p, _p, _i, _i, _i, _p]),

@@ -9,10 +9,11 @@
 //
 // Recurrence (vmx_gated_delta_rule), per head with a matrix memory S [dim, vdim] in f32:
 //   S <- diag(g_t) S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
-// so a token reads the memory after its own write.  Query/key head of value head h: h / (heads / qk_heads).  A workgroup owns 32
-// value columns of one (sequence, head) and walks the sequence's tokens of the step in order; 8 threads share a column, each
-// holding every 8th row of S in registers, and the two column sums per token are 8-lane butterflies.  The state slot keeps S in
-// the workgroup's own register order (the layout is private to this kernel), so that loading and storing it is coalesced.
+// so a token reads the memory after its own write (computed as (g S)^T q + u (k . q), the same sum in another order).  Query/key
+// head of value head h: h / (heads / qk_heads).  A workgroup owns 16 value columns of one (sequence, head) and walks the
+// sequence's tokens of the step in order; 16 threads share a column, each holding every 16th row of S in registers, and the
+// column sums per token are 16-lane butterflies.  The state slot keeps S in the workgroup's own register order (the layout is
+// private to this kernel), so that loading and storing it is coalesced.
 #include "vmx_kernels.h"
 
 namespace {
@@ -49,8 +50,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const ConvArgs a) 
     const int first = a.seq_starts[seq];             // packed row of the sequence's first token in this step
     const int start = pos - (t - first);             // position of that token
     const float *st = a.state + (int64_t)a.state_slots[seq] * (a.n - 1) * a.channels;
-    float ss = 0.f;
-    for (int c = c0 + lane; c < c1; c += 64) {
+    auto conv_at = [&](int c) {
         float acc = 0.f;
         for (int s = a.n - 1; s >= 0; s--) {         // oldest input first
             const int q = pos - s;
@@ -58,15 +58,30 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const ConvArgs a) 
             const float xv = q >= start ? a.x[(int64_t)(t - s) * a.ldx + c] : st[(int64_t)(q - start + a.n - 1) * a.channels + c];
             acc = fmaf(vmx_bf16_to_f32(a.taps[(int64_t)c * a.n + (a.n - 1 - s)]), xv, acc);
         }
-        const float yv = silu_f(acc);
+        return silu_f(acc);
+    };
+    constexpr int HOLD = 4;                          // a lane's outputs of a run of up to 256 channels stay in registers
+    float held[HOLD], ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < HOLD; i++) {
+        const int c = c0 + lane + 64 * i;
+        held[i] = c < c1 ? conv_at(c) : 0.f;
+        ss = fmaf(held[i], held[i], ss);
+    }
+    for (int c = c0 + lane + 64 * HOLD; c < c1; c += 64) {   // wider runs go through memory
+        const float yv = conv_at(c);
         a.y[(int64_t)t * a.ldy + c] = yv;
         ss = fmaf(yv, yv, ss);
     }
-    if (unit) {
-        ss = vmx_wave_sum(ss);
-        const float f = (run < a.scaled_groups ? a.mul : 1.0f) / sqrtf(ss + a.unit_eps);
-        for (int c = c0 + lane; c < c1; c += 64) a.y[(int64_t)t * a.ldy + c] *= f;   // each lane rescales what it wrote itself
+    float f = 1.0f;
+    if (unit) f = (run < a.scaled_groups ? a.mul : 1.0f) / sqrtf(vmx_wave_sum(ss) + a.unit_eps);
+#pragma unroll
+    for (int i = 0; i < HOLD; i++) {
+        const int c = c0 + lane + 64 * i;
+        if (c < c1) a.y[(int64_t)t * a.ldy + c] = held[i] * f;
     }
+    if (unit)
+        for (int c = c0 + lane + 64 * HOLD; c < c1; c += 64) a.y[(int64_t)t * a.ldy + c] *= f;   // each lane rescales what it wrote itself
 }
 
 // state[slot] <- the last n - 1 inputs of the sequence after this step.  A thread owns one (sequence, channel) and goes through
@@ -111,16 +126,25 @@ struct DeltaArgs {
     int heads, qk_heads, dim, vdim;
 };
 
-constexpr int DR_RS = 8, DR_VT = 32, DR_CT = 8;   // row splits per column, columns per workgroup, tokens staged per round
+constexpr int DR_RS = 16, DR_VT = 16;   // row splits per column, columns per workgroup
 
+// Tokens are staged in rounds of CT through two LDS buffers: the next round is requested into registers before the current one
+// is walked and stored afterwards, so one barrier per round remains and the walk never waits for memory.  q, k and g are stored
+// in thread order ([row split r][u] for row r + 8 u), so a thread reads its rows as 16-byte vectors.
 template <int DPT>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a) {
     constexpr int DP = DPT * DR_RS;          // padded key dimension
-    __shared__ float sq[DR_CT][DP], sk[DR_CT][DP], sg[DR_CT][DP], sv[DR_CT][DR_VT], sb[DR_CT];
+    constexpr int LDP = DPT == 4 ? 4 : DPT + 4;   // floats between two row splits in LDS: the 16 splits of a read fall on different banks
+    constexpr int CT = 128 / DPT;            // tokens per round: long enough for the next round's loads to land while this one is walked
+    constexpr int NL = CT * DP / 256;        // q / k / g elements a thread stages per round
+    constexpr int NV = (CT * DR_VT + 255) / 256;
+    constexpr int ROW = DR_RS * LDP;         // floats of one token's q (k, g) in LDS
+    extern __shared__ __align__(16) float delta_lds[];   // delta_lds_bytes(DPT): q | k | g [2][CT][ROW], v [2][CT][16], beta [2][CT]
+    float *sq = delta_lds, *sk = sq + 2 * CT * ROW, *sg = sk + 2 * CT * ROW, *sv = sg + 2 * CT * ROW, *sb = sv + 2 * CT * DR_VT;
     const int seq = blockIdx.z, h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
     const int first = a.seq_starts[seq], count = a.seq_starts[seq + 1] - first;
     if (count <= 0) return;
-    const int r = tid & (DR_RS - 1), cl = tid >> 3, c = tile * DR_VT + cl;
+    const int r = tid & (DR_RS - 1), cl = tid >> 4, c = tile * DR_VT + cl;
     const int qh = h / (a.heads / a.qk_heads);
     const int tiles = gridDim.x;
     float *sp = a.state + ((((int64_t)a.state_slots[seq] * a.heads + h) * tiles + tile) * DPT) * 256 + tid;
@@ -128,46 +152,94 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const DeltaArgs a
     const bool fresh = a.positions[first] == 0;
 #pragma unroll
     for (int u = 0; u < DPT; u++) S[u] = fresh ? 0.f : sp[(int64_t)u * 256];
-    for (int t0 = 0; t0 < count; t0 += DR_CT) {
-        const int ct = min(DR_CT, count - t0);
-        __syncthreads();
-        for (int i = tid; i < ct * DP; i += 256) {
-            const int tt = i / DP, d = i % DP;
+    float rq[NL], rk[NL], rg[NL], rv[NV], rb = 0.f;
+    auto request = [&](int t0) {
+        const int ct = min(CT, count - t0);
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            const int i = tid + 256 * j, tt = i / DP, d = i % DP;
             const int64_t row = first + t0 + tt;
-            const bool in = d < a.dim;
-            sq[tt][d] = in ? a.q[row * a.ldq + (int64_t)qh * a.dim + d] : 0.f;
-            sk[tt][d] = in ? a.k[row * a.ldk + (int64_t)qh * a.dim + d] : 0.f;
-            sg[tt][d] = in ? a.g[row * a.ldg + (int64_t)h * a.dim + d] : 1.f;
+            const bool in = tt < ct && d < a.dim;
+            rq[j] = in ? a.q[row * a.ldq + (int64_t)qh * a.dim + d] : 0.f;
+            rk[j] = in ? a.k[row * a.ldk + (int64_t)qh * a.dim + d] : 0.f;
+            rg[j] = in ? a.g[row * a.ldg + (int64_t)h * a.dim + d] : 1.f;
         }
-        for (int i = tid; i < ct * DR_VT; i += 256) {
-            const int tt = i / DR_VT, cc = tile * DR_VT + i % DR_VT;
-            sv[tt][i % DR_VT] = cc < a.vdim ? a.v[(int64_t)(first + t0 + tt) * a.ldv + (int64_t)h * a.vdim + cc] : 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = tid + 256 * j, tt = i / DR_VT, cc = tile * DR_VT + i % DR_VT;
+            rv[j] = (tt < ct && cc < a.vdim) ? a.v[(int64_t)(first + t0 + tt) * a.ldv + (int64_t)h * a.vdim + cc] : 0.f;
         }
-        if (tid < ct) sb[tid] = a.beta[(int64_t)(first + t0 + tid) * a.ldbeta + h];
+        rb = tid < ct ? a.beta[(int64_t)(first + t0 + tid) * a.ldbeta + h] : 0.f;
+    };
+    auto stage = [&](int b) {
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            const int i = tid + 256 * j, tt = i / DP, d = i % DP, at = (d & (DR_RS - 1)) * LDP + (d >> 4);   // row d = r + 16 u -> [r][u]
+            sq[(b * CT + tt) * ROW + at] = rq[j];
+            sk[(b * CT + tt) * ROW + at] = rk[j];
+            sg[(b * CT + tt) * ROW + at] = rg[j];
+        }
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = tid + 256 * j;
+            if (i < CT * DR_VT) sv[b * CT * DR_VT + i] = rv[j];
+        }
+        if (tid < CT) sb[b * CT + tid] = rb;
+    };
+    request(0);
+    stage(0);
+    __syncthreads();
+    int b = 0;
+    for (int t0 = 0; t0 < count; t0 += CT, b ^= 1) {
+        const int ct = min(CT, count - t0);
+        const bool more = t0 + CT < count;
+        if (more) request(t0 + CT);
+        // The read-out is taken from the decayed memory: o = (gS)^T q + u (k . q), so the three column sums of a token, (gS)^T k,
+        // (gS)^T q and k . q, are independent chains and the write S += k u^T leaves the critical path.  The LDS reads of the next
+        // token are issued before the current one is worked on (two register sets, A and B).
+        auto ld = [&](int tt, float (&kk)[DPT], float (&gg)[DPT], float (&qq)[DPT], float &bv, float &vv) {
+#pragma unroll
+            for (int u = 0; u < DPT; u += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(sk + (b * CT + tt) * ROW + r * LDP + u);
+                const float4 g4 = *reinterpret_cast<const float4 *>(sg + (b * CT + tt) * ROW + r * LDP + u);
+                const float4 q4 = *reinterpret_cast<const float4 *>(sq + (b * CT + tt) * ROW + r * LDP + u);
+                kk[u] = k4.x, kk[u + 1] = k4.y, kk[u + 2] = k4.z, kk[u + 3] = k4.w;
+                gg[u] = g4.x, gg[u + 1] = g4.y, gg[u + 2] = g4.z, gg[u + 3] = g4.w;
+                qq[u] = q4.x, qq[u + 1] = q4.y, qq[u + 2] = q4.z, qq[u + 3] = q4.w;
+            }
+            bv = sb[b * CT + tt];
+            vv = sv[(b * CT + tt) * DR_VT + cl];
+        };
+        auto step = [&](int tt, const float (&kk)[DPT], const float (&gg)[DPT], const float (&qq)[DPT], float bv, float vv) {
+            float pk = 0.f, pq = 0.f, kq = 0.f;
+#pragma unroll
+            for (int u = 0; u < DPT; u++) {
+                S[u] *= gg[u];
+                pk = fmaf(S[u], kk[u], pk);
+                pq = fmaf(S[u], qq[u], pq);
+                kq = fmaf(kk[u], qq[u], kq);
+            }
+            pk += vmx_dpp<VMX_DPP_XOR1>(pk), pq += vmx_dpp<VMX_DPP_XOR1>(pq), kq += vmx_dpp<VMX_DPP_XOR1>(kq);
+            pk += vmx_dpp<VMX_DPP_XOR2>(pk), pq += vmx_dpp<VMX_DPP_XOR2>(pq), kq += vmx_dpp<VMX_DPP_XOR2>(kq);
+            pk += vmx_dpp<VMX_DPP_HALF_MIRROR>(pk), pq += vmx_dpp<VMX_DPP_HALF_MIRROR>(pq), kq += vmx_dpp<VMX_DPP_HALF_MIRROR>(kq);
+            pk += vmx_dpp<VMX_DPP_ROR8>(pk), pq += vmx_dpp<VMX_DPP_ROR8>(pq), kq += vmx_dpp<VMX_DPP_ROR8>(kq);
+            const float uu = bv * (vv - pk);
+            if (r == 0 && c < a.vdim) a.o[(int64_t)(first + t0 + tt) * a.ldo + (int64_t)h * a.vdim + c] = fmaf(uu, kq, pq);
+#pragma unroll
+            for (int u = 0; u < DPT; u++) S[u] = fmaf(kk[u], uu, S[u]);
+        };
+        float kA[DPT], gA[DPT], qA[DPT], kB[DPT], gB[DPT], qB[DPT], bA, vA, bB = 0.f, vB = 0.f;
+        ld(0, kA, gA, qA, bA, vA);
+        for (int tt = 0; tt < ct; tt += 2) {
+            if (tt + 1 < ct) ld(tt + 1, kB, gB, qB, bB, vB);
+            step(tt, kA, gA, qA, bA, vA);
+            if (tt + 1 < ct) {
+                if (tt + 2 < ct) ld(tt + 2, kA, gA, qA, bA, vA);
+                step(tt + 1, kB, gB, qB, bB, vB);
+            }
+        }
+        if (more) stage(b ^ 1);
         __syncthreads();
-        for (int tt = 0; tt < ct; tt++) {
-            float kk[DPT], part = 0.f;
-#pragma unroll
-            for (int u = 0; u < DPT; u++) {
-                kk[u] = sk[tt][r + DR_RS * u];
-                S[u] *= sg[tt][r + DR_RS * u];
-                part = fmaf(S[u], kk[u], part);
-            }
-            part += vmx_dpp<VMX_DPP_XOR1>(part);
-            part += vmx_dpp<VMX_DPP_XOR2>(part);
-            part += vmx_dpp<VMX_DPP_HALF_MIRROR>(part);
-            const float uu = sb[tt] * (sv[tt][cl] - part);
-            float po = 0.f;
-#pragma unroll
-            for (int u = 0; u < DPT; u++) {
-                S[u] = fmaf(kk[u], uu, S[u]);
-                po = fmaf(S[u], sq[tt][r + DR_RS * u], po);
-            }
-            po += vmx_dpp<VMX_DPP_XOR1>(po);
-            po += vmx_dpp<VMX_DPP_XOR2>(po);
-            po += vmx_dpp<VMX_DPP_HALF_MIRROR>(po);
-            if (r == 0 && c < a.vdim) a.o[(int64_t)(first + t0 + tt) * a.ldo + (int64_t)h * a.vdim + c] = po;
-        }
     }
 #pragma unroll
     for (int u = 0; u < DPT; u++) sp[(int64_t)u * 256] = S[u];
@@ -246,7 +318,21 @@ extern "C" int vmx_delta_rule_gates(float *g, int64_t ldg, const uint16_t *a_log
     return VMX_OK;
 }
 
-static int delta_dpt(int dim) { return dim <= 64 ? 8 : (dim <= 128 ? 16 : 32); }
+static int delta_dpt(int dim) { return dim <= 64 ? 4 : (dim <= 128 ? 8 : 16); }
+static size_t delta_lds_bytes(int dpt) {
+    const size_t ct = 128 / dpt, row = (size_t)DR_RS * (dpt == 4 ? 4 : dpt + 4);
+    return (3 * 2 * ct * row + 2 * ct * DR_VT + 2 * ct) * 4;
+}
+template <int DPT> static int delta_launch(const DeltaArgs &a, dim3 grid, hipStream_t st) {
+    static bool sized = false;   // more than 64 KiB of LDS has to be asked for once per kernel
+    const size_t lds = delta_lds_bytes(DPT);
+    if (!sized) {
+        VMX_CHECK_HIP(hipFuncSetAttribute((const void *)gated_delta_rule_kernel<DPT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        sized = true;
+    }
+    hipLaunchKernelGGL(gated_delta_rule_kernel<DPT>, grid, dim3(256), lds, st, a);
+    return VMX_OK;
+}
 
 extern "C" size_t vmx_gated_delta_rule_state_bytes(int slots, int heads, int dim, int vdim) {
     const size_t tiles = (vdim + DR_VT - 1) / DR_VT;
@@ -263,13 +349,15 @@ extern "C" int vmx_gated_delta_rule(float *o, int64_t ldo, const float *q, int64
     VMX_REQUIRE(dim >= 1 && dim <= 256 && vdim >= 1, "gated_delta_rule: key size %d outside 1..256", dim);
     if (num_seqs <= 0) return VMX_OK;
     const DeltaArgs a{q, k, v, g, beta, ldq, ldk, ldv, ldg, ldbeta, o, ldo, state, positions, seq_starts, state_slots, heads, qk_heads, dim, vdim};
-    const dim3 grid((vdim + DR_VT - 1) / DR_VT, heads, num_seqs), block(256);
+    const dim3 grid((vdim + DR_VT - 1) / DR_VT, heads, num_seqs);
     hipStream_t st = vmx_stream(stream);
+    int rc;
     switch (delta_dpt(dim)) {
-        case 8: hipLaunchKernelGGL(gated_delta_rule_kernel<8>, grid, block, 0, st, a); break;
-        case 16: hipLaunchKernelGGL(gated_delta_rule_kernel<16>, grid, block, 0, st, a); break;
-        default: hipLaunchKernelGGL(gated_delta_rule_kernel<32>, grid, block, 0, st, a); break;
+        case 4: rc = delta_launch<4>(a, grid, st); break;
+        case 8: rc = delta_launch<8>(a, grid, st); break;
+        default: rc = delta_launch<16>(a, grid, st); break;
     }
+    if (rc) return rc;
     VMX_CHECK_LAUNCH("gated_delta_rule");
     return VMX_OK;
 }

@@ -53,7 +53,7 @@ struct vmx_gupuvik {
     std::vector<Layer> layers;
     Buf embed, final_norm, head;
     std::vector<std::string> missing;
-    Buf x, h, hsel, fused, attn, conv, dec, gate2, dro, argmax_keys, few_pairs, rlogits, topw, topi, sorted, blk_expert, total, inv, gu, act, ydown;
+    Buf x, h, hsel, fused, attn, attn_ws, conv, dec, gate2, dro, argmax_keys, few_pairs, rlogits, topw, topi, sorted, blk_expert, total, inv, gu, act, ydown;
     bool f32() const { return cfg.dtype == VMX_F32; }
     size_t esz() const { return f32() ? 4 : 2; }
 };
@@ -94,7 +94,7 @@ extern "C" int vmx_gupuvik_create(const vmx_gupuvik_config *cfg, const vmx_gupuv
     m->cfg = c;
     m->layers.resize(c.num_layers);
     const size_t T = c.max_tokens, W = c.width, rows = (size_t)c.num_blocks * c.block_size;
-    size_t nf = 8, hv = 1, convc = 1, hd = 1, ne = 1, pairs = 0, cap = (size_t)VMX_MOE_FEW_PAIRS * 16, eff = 1, actn = 1;
+    size_t attn_ws = 16, nf = 8, hv = 1, convc = 1, hd = 1, ne = 1, pairs = 0, cap = (size_t)VMX_MOE_FEW_PAIRS * 16, eff = 1, actn = 1;
     int rc = VMX_OK;
 #define GA(buf, n)                        \
     do {                                  \
@@ -152,6 +152,7 @@ extern "C" int vmx_gupuvik_create(const vmx_gupuvik_config *cfg, const vmx_gupuv
                 L.want("mix.v", &L.wfused, (size_t)L.v_off * W * 2, G * V * W * 2);
                 L.want("mix.v.b", &L.bias, (size_t)L.v_off * 2, G * V * 2);
             }
+            attn_ws = std::max(attn_ws, vmx_window_attention_workspace_bytes((int)T, lc.heads, lc.vdim));
             L.want("mix.temp", &L.temp, 0, H * 2);
             L.want("mix.g", &L.wfused, (size_t)L.g_off * W * 2, H * W * 2);
             L.want("mix.o", &L.wo, 0, W * H * V * 2);
@@ -250,6 +251,7 @@ extern "C" int vmx_gupuvik_create(const vmx_gupuvik_config *cfg, const vmx_gupuv
     GA(m->hsel, T * W * m->esz());
     GA(m->fused, T * std::max(nf, (size_t)c.vocab) * 4);   // also the logits of a greedy-only step
     GA(m->attn, T * hv * m->esz());
+    GA(m->attn_ws, attn_ws);   // key shares of attention launches with few rows
     GA(m->conv, T * convc * 4);
     GA(m->dec, T * hd * 4);
     GA(m->gate2, T * hv * 4);
@@ -296,7 +298,7 @@ extern "C" void vmx_gupuvik_destroy(vmx_gupuvik *m) {
         for (Buf *b : {&L.norm1, &L.wfused, &L.bias, &L.wo, &L.temp, &L.kcache, &L.vcache, &L.conv_taps, &L.a_log, &L.dt_bias, &L.onorm, &L.wa2, &L.wg2,
                        &L.conv_state, &L.s_state, &L.wup, &L.wdown, &L.router, &L.egu, &L.edown})
             b->release();
-    for (Buf *b : {&m->embed, &m->final_norm, &m->head, &m->x, &m->h, &m->hsel, &m->fused, &m->attn, &m->conv, &m->dec, &m->gate2, &m->dro,
+    for (Buf *b : {&m->embed, &m->final_norm, &m->head, &m->x, &m->h, &m->hsel, &m->fused, &m->attn, &m->attn_ws, &m->conv, &m->dec, &m->gate2, &m->dro,
                    &m->argmax_keys, &m->few_pairs, &m->rlogits, &m->topw, &m->topi, &m->sorted, &m->blk_expert, &m->total, &m->inv, &m->gu, &m->act,
                    &m->ydown})
         b->release();
@@ -384,7 +386,7 @@ extern "C" int vmx_gupuvik_forward(vmx_gupuvik *m, const int32_t *tokens, const 
             Layer &S = lc.kv_from < 0 ? L : m->layers[lc.kv_from];
             if (int rc = vmx_window_attention(m->attn.p, cdt, fused + L.q_off, nf, S.kcache.p, S.vcache.p, cdt, block_tables, max_blocks_per_seq,
                                               seq_ids, positions, L.temp.as<uint16_t>(), fused + L.g_off, nf, lc.scale, lc.softcap, lc.window,
-                                              lc.keep_first, T, H, G, D, V, c.block_size, seq_starts, num_seqs, st))
+                                              lc.keep_first, T, H, G, D, V, c.block_size, seq_starts, num_seqs, m->attn_ws.p, m->attn_ws.bytes, st))
                 return rc;
         } else {
             const int C = 2 * G * D + H * V;

@@ -13,6 +13,7 @@
 // key l of the tile, then every lane sums its value columns) and the matrix-core form below for bf16 caches.
 #include "vmx_kernels.h"
 #include <float.h>
+#include <algorithm>
 
 namespace {
 
@@ -39,6 +40,9 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(const float *__rest
     }
 }
 
+// tanh through one exponential, for the bf16 matrix-core form: absolute error about 1e-7, far below the bf16 rounding of its operands
+__device__ __forceinline__ float tanh_fast(float y) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * y)); }
+
 struct WinAttn {
     void *out;
     int out_f32;
@@ -54,6 +58,9 @@ struct WinAttn {
     int window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size;
     const int32_t *seq_starts;   // matrix-core form: sequence s owns the packed rows seq_starts[s] .. seq_starts[s + 1] - 1
     int num_seqs;
+    int bs_shift;                // log2(block_size) when it is a power of two, else -1
+    int parts;                   // > 1: the key tiles of a run are dealt to `parts` workgroups, whose results go to `ws` for the merge
+    float *ws;                   // [tokens, heads, parts, vdim + 2]: unnormalised sums, running maximum, denominator
 };
 
 constexpr int WA_MAX_DIM = 256;
@@ -141,7 +148,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
     __shared__ __align__(16) uint16_t Vt[16 * VS * LDV];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fl = lane & 15, fg = lane >> 4;
     const int qpk = p.heads / p.kv_heads, hq = min(qpk, 4), nt = 4 / hq, RT = 16 * nt;
-    int tile = blockIdx.x, r0 = 0, nrows = 0;
+    const int share = blockIdx.x % p.parts;
+    int tile = blockIdx.x / p.parts, r0 = 0, nrows = 0;
     for (int s = 0; s < p.num_seqs; s++) {
         const int a = p.seq_starts[s], len = p.seq_starts[s + 1] - a, n = (len + RT - 1) / RT;
         if (tile < n) {
@@ -180,24 +188,36 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
     }
     const float smul = p.scale * (p.temp ? vmx_bf16_to_f32(p.temp[head]) : 1.0f);
     const float inv_cap = p.softcap > 0.f ? 1.0f / p.softcap : 0.f;
+    // this workgroup's share of the run's key tiles
+    const int ntile = (nk + KT - 1) / KT, per = (ntile + p.parts - 1) / p.parts;
+    const int kb0 = share * per * KT, kb1 = min(nk, (share + 1) * per * KT);
     uint4 kr[KCH], vr[VCH];
-    auto cache_row = [&](int idx) -> int64_t {
+    int krow[KCH], vrow[VCH];    // cache rows of the tile to fetch next: looked up one tile earlier, so that a fetch is one trip to memory
+    auto cache_row = [&](int idx) -> int {
+        if (idx >= nk) return 0;
         const int j = idx < na ? idx : lo + (idx - na);
-        return (int64_t)bt[j / p.block_size] * p.block_size + j % p.block_size;
+        if (p.bs_shift >= 0) return (bt[j >> p.bs_shift] << p.bs_shift) + (j & (p.block_size - 1));
+        return bt[j / p.block_size] * p.block_size + j % p.block_size;
+    };
+    auto lookup = [&](int kb) {
+#pragma unroll
+        for (int c = 0; c < KCH; c++) krow[c] = cache_row(kb + (tid + 256 * c) / (4 * DS));
+#pragma unroll
+        for (int c = 0; c < VCH; c++) vrow[c] = cache_row(kb + (tid + 256 * c) % KT);
     };
     auto fetch = [&](int kb) {
 #pragma unroll
         for (int c = 0; c < KCH; c++) {
             const int ch = tid + 256 * c, kk = ch / (4 * DS), part = ch % (4 * DS);
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (kb + kk < nk && 8 * part < D) v = *reinterpret_cast<const uint4 *>(kc + cache_row(kb + kk) * kw + (int64_t)kvh * D + 8 * part);
+            if (kb + kk < kb1 && 8 * part < D) v = *reinterpret_cast<const uint4 *>(kc + (int64_t)krow[c] * kw + (int64_t)kvh * D + 8 * part);
             kr[c] = v;
         }
 #pragma unroll
         for (int c = 0; c < VCH; c++) {
-            const int ch = tid + 256 * c, kk = ch / (2 * VS), part = ch % (2 * VS);
+            const int ch = tid + 256 * c, kk = ch % KT, part = ch / KT;   // a wave's lanes: 64 keys, so that their LDS columns differ
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (ch < KT * 2 * VS && kb + kk < nk && 8 * part < V) v = *reinterpret_cast<const uint4 *>(vc + cache_row(kb + kk) * vw + (int64_t)kvh * V + 8 * part);
+            if (ch < KT * 2 * VS && kb + kk < kb1 && 8 * part < V) v = *reinterpret_cast<const uint4 *>(vc + (int64_t)vrow[c] * vw + (int64_t)kvh * V + 8 * part);
             vr[c] = v;
         }
     };
@@ -209,7 +229,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
         }
 #pragma unroll
         for (int c = 0; c < VCH; c++) {
-            const int ch = tid + 256 * c, kk = ch / (2 * VS), part = ch % (2 * VS);
+            const int ch = tid + 256 * c, kk = ch % KT, part = ch / KT;
             if (ch < KT * 2 * VS) {
                 // key kk of the tile sits in k slot `col`: the order in which the score registers of a lane line up as an operand
                 const int col = 32 * (kk >> 5) + 8 * ((kk & 15) >> 2) + (kk & 3) + 4 * ((kk >> 4) & 1);
@@ -223,11 +243,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
     vmx_f32x4 o[VS];
 #pragma unroll
     for (int v = 0; v < VS; v++) o[v] = vmx_f32x4{0.f, 0.f, 0.f, 0.f};
-    fetch(0);
+    lookup(kb0);
+    fetch(kb0);
+    lookup(kb0 + KT);
     stash();
     __syncthreads();
-    for (int kb = 0; kb < nk; kb += KT) {
-        if (kb + KT < nk) fetch(kb + KT);
+    for (int kb = kb0; kb < kb1; kb += KT) {
+        if (kb + KT < kb1) {
+            fetch(kb + KT);
+            lookup(kb + 2 * KT);
+        }
         if (active) {
             float sc[4][4];
             float tmax = -FLT_MAX;
@@ -243,9 +268,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
                 for (int r = 0; r < 4; r++) {
                     const int idx = kb + 16 * kt + 4 * fg + r;
                     const int j = idx < na ? idx : lo + (idx - na);
-                    const bool vis = qlive && idx < nk && j <= qi && (p.window == 0 || qi - j < p.window || j < p.keep_first);
+                    const bool vis = qlive && idx < kb1 && j <= qi && (p.window == 0 || qi - j < p.window || j < p.keep_first);
                     float x = acc[r] * smul;
-                    if (p.softcap > 0.f) x = p.softcap * tanhf(x * inv_cap);
+                    if (p.softcap > 0.f) x = p.softcap * tanh_fast(x * inv_cap);
                     sc[kt][r] = vis ? x : -FLT_MAX;
                     tmax = fmaxf(tmax, sc[kt][r]);
                 }
@@ -253,23 +278,25 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
             tmax = fmaxf(tmax, vmx_lane_xor<16>(tmax));
             tmax = fmaxf(tmax, vmx_lane_xor<32>(tmax));
             const float mn = fmaxf(m, tmax);
-            const float f = expf(m - mn);
+            const float f = __expf(m - mn);
             float psum = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; kt++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    sc[kt][r] = sc[kt][r] > -FLT_MAX ? expf(sc[kt][r] - mn) : 0.f;
+                    sc[kt][r] = sc[kt][r] > -FLT_MAX ? __expf(sc[kt][r] - mn) : 0.f;
                     psum += sc[kt][r];
                 }
             psum += vmx_lane_xor<16>(psum);
             psum += vmx_lane_xor<32>(psum);
             den = den * f + psum;
             m = mn;
+            if (__any(f != 1.0f)) {   // the maximum of some row moved: rescale what was summed so far
 #pragma unroll
-            for (int v = 0; v < VS; v++)
+                for (int v = 0; v < VS; v++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) o[v][r] *= f;
+                    for (int r = 0; r < 4; r++) o[v][r] *= f;
+            }
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 float hi[8], lw[8];
@@ -289,12 +316,24 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
             }
         }
         __syncthreads();
-        if (kb + KT < nk) {
+        if (kb + KT < kb1) {
             stash();
             __syncthreads();
         }
     }
     if (!qlive) return;
+    if (p.parts > 1) {           // this share's sums as they are; the merge kernel normalises
+        float *w = p.ws + (((int64_t)(r0 + qrow) * p.heads + head) * p.parts + share) * (V + 2);
+#pragma unroll
+        for (int v = 0; v < VS; v++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int c = 16 * v + 4 * fg + r;
+                if (c < V) w[c] = o[v][r];
+            }
+        if (fg == 0) w[V] = m, w[V + 1] = den;
+        return;
+    }
     float g = 1.0f / den;
     if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)(r0 + qrow) * p.ldgate + head]));
 #pragma unroll
@@ -310,7 +349,38 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(const WinAttn p) 
         }
 }
 
+// out[t, h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) den_p * sigmoid(gate): the shares of a row's keys put together.  One wave
+// per row: lane p takes share p's maximum and denominator (at most 16 shares), the weights are then handed round by lane reads.
+__global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) {
+    const int row = blockIdx.x, t = row / p.heads, h = row % p.heads, V = p.vdim, lane = threadIdx.x;
+    const float *w = p.ws + (int64_t)row * p.parts * (V + 2);
+    const bool mine = lane < p.parts;
+    const float mq = mine ? w[lane * (V + 2) + V] : -FLT_MAX, dq = mine ? w[lane * (V + 2) + V + 1] : 0.f;
+    const float M = vmx_wave_max(mq);
+    const float eq = mine ? expf(mq - M) : 0.f;            // a share without keys: e^(-huge) = 0
+    float g = 1.0f / vmx_wave_sum(eq * dq);
+    if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)t * p.ldgate + h]));
+    for (int c0 = 0; c0 < V; c0 += 64) {
+        const int c = c0 + lane;
+        float acc = 0.f;
+        for (int q = 0; q < p.parts; q++) {
+            const float e = __shfl(eq, q, 64);
+            if (c < V) acc = fmaf(e, w[q * (V + 2) + c], acc);
+        }
+        if (c < V) {
+            const int64_t at = (int64_t)row * V + c;
+            if (p.out_f32) ((float *)p.out)[at] = acc * g;
+            else ((uint16_t *)p.out)[at] = vmx_f32_to_bf16(acc * g);
+        }
+    }
+}
+
 }  // namespace
+
+extern "C" size_t vmx_window_attention_workspace_bytes(int tokens, int heads, int vdim) {
+    // enough for 16 shares of up to 256 rows: launches with more rows fill the chip without splitting their keys
+    return (size_t)(tokens < 256 ? tokens : 256) * heads * 16 * (vdim + 2) * 4;
+}
 
 extern "C" int vmx_kv_cache_write_f32(const float *k, int64_t ldk, const float *v, int64_t ldv, const int32_t *slots, void *k_cache,
                                       void *v_cache, int cache_dtype, int tokens, int k_width, int v_width, void *stream) {
@@ -328,7 +398,8 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
                                     int cache_dtype, const int32_t *block_tables, int max_blocks_per_seq, const int32_t *seq_ids,
                                     const int32_t *positions, const uint16_t *head_temp_bf16, const float *gate, int64_t ldgate, float scale,
                                     float softcap, int window, int keep_first, int tokens, int heads, int kv_heads, int dim, int vdim,
-                                    int block_size, const int32_t *seq_starts, int num_seqs, void *stream) {
+                                    int block_size, const int32_t *seq_starts, int num_seqs, void *workspace, size_t workspace_bytes,
+                                    void *stream) {
     VMX_REQUIRE(out && q && k_cache && v_cache && block_tables && seq_ids && positions, "window_attention: null pointer");
     VMX_REQUIRE((out_dtype == VMX_F32 || out_dtype == VMX_BF16) && (cache_dtype == VMX_F32 || cache_dtype == VMX_BF16),
                 "window_attention: f32 or bf16 output and cache");
@@ -339,13 +410,22 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
     VMX_REQUIRE(ldq >= (int64_t)heads * dim && (!gate || ldgate >= heads), "window_attention: bad row strides");
     if (tokens <= 0) return VMX_OK;
     WinAttn p{out, out_dtype == VMX_F32, q, ldq, k_cache, v_cache, block_tables, seq_ids, positions, max_blocks_per_seq, head_temp_bf16,
-              gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size, seq_starts, num_seqs};
+              gate, ldgate, scale, softcap, window, keep_first, tokens, heads, kv_heads, dim, vdim, block_size, seq_starts, num_seqs,
+              (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1, 1, (float *)workspace};
     hipStream_t st = vmx_stream(stream);
     const bool f32 = cache_dtype == VMX_F32;
     if (!f32 && seq_starts && num_seqs >= 1 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 128 && ldq % 4 == 0 && ((uintptr_t)q & 15) == 0 &&
         ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)v_cache & 15) == 0) {
         const int qpk = heads / kv_heads, hq = qpk < 4 ? qpk : 4, rt = 16 * (4 / hq);
-        const dim3 mgrid(tokens / rt + num_seqs, kv_heads, (qpk + 3) / 4);   // at most one partly filled run per sequence
+        const int runs = tokens / rt + num_seqs;                              // at most one partly filled run per sequence
+        const int base = runs * kv_heads * ((qpk + 3) / 4);
+        if (workspace && base < 128) {   // few workgroups: deal each run's key tiles to several
+            int parts = 256 / base < 16 ? 256 / base : 16;
+            if (window > 0) parts = std::min(parts, (window + keep_first + rt + 63) / 64);
+            parts = std::min<size_t>(parts, workspace_bytes / ((size_t)tokens * heads * (vdim + 2) * 4));
+            if (parts > 1) p.parts = parts;
+        }
+        const dim3 mgrid(runs * p.parts, kv_heads, (qpk + 3) / 4);
         const int ds = dim <= 64 ? 2 : (dim <= 128 ? 4 : 8), vs = vdim <= 32 ? 2 : (vdim <= 64 ? 4 : 8);
 #define WM_LAUNCH(A, B) hipLaunchKernelGGL((window_attn_mfma_kernel<A, B>), mgrid, dim3(256), 0, st, p)
         if (ds == 2) {
@@ -362,6 +442,7 @@ extern "C" int vmx_window_attention(void *out, int out_dtype, const float *q, in
             else WM_LAUNCH(8, 8);
         }
 #undef WM_LAUNCH
+        if (p.parts > 1) hipLaunchKernelGGL(window_attn_merge_kernel, dim3(tokens * heads), dim3(64), 0, st, p);
         VMX_CHECK_LAUNCH("window_attention (matrix cores)");
         return VMX_OK;
     }
