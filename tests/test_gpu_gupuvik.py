@@ -584,3 +584,24 @@ def test_trace_replay_tool(gpu, tmp_path):
     rd = lambda i: np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, spec.vocab)   # noqa: E731
     assert rel_err(rd(0), np.stack([wa[0], wa[8], wb[5]])) <= TOL["float32"]
     assert rel_err(rd(1), wb[6:7]) <= TOL["float32"] and rel_err(rd(2), wa[10:11]) <= TOL["float32"] and rel_err(rd(3), wa[11:12]) <= TOL["float32"]
+
+
+def test_generation_tool(gpu, tmp_path):
+    """bin/generate as a subprocess (registry, scheduler, greedy ids from the executor) against greedy decoding with the oracle."""
+    vmx, torch = gpu
+    spec = small_spec()
+    w = _write_checkpoint(tmp_path, spec, 8)
+    prompts = [tokens_for(spec, 9, 3), tokens_for(spec, 2, 4)]
+    p = subprocess.run([sys.executable, str(ROOT / "bin" / "generate"), "--model", str(tmp_path), "--dtype", "float32", "--max-new-tokens", "4",
+                        "--max-tokens", "64", "--prefill-chunk", "4"] + [a for q in prompts for a in ("--prompt", ",".join(map(str, q)))],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    outs = [[int(t) for t in line.split(",")] for line in p.stdout.strip().splitlines()]
+    assert len(outs) == 2
+    for q, got in zip(prompts, outs):
+        seq = list(q)
+        for t in got:
+            lg = oracle_logits(spec, w, seq)[-1]
+            top2 = np.sort(lg)[-2:]
+            assert int(np.argmax(lg)) == t or top2[1] - top2[0] < 1e-3 * (np.abs(lg).max() + 1e-9)
+            seq.append(t)
