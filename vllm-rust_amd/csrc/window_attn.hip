@@ -361,12 +361,13 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const WinAttn p) 
     float g = 1.0f / vmx_wave_sum(eq * dq);
     if (p.gate) g *= 1.0f / (1.0f + expf(-p.gate[(int64_t)t * p.ldgate + h]));
     for (int c0 = 0; c0 < V; c0 += 64) {
-        const int c = c0 + lane;
+        const int c = c0 + lane, cc = min(c, V - 1);
+        float x[16];                                       // every share's value first: independent loads, one wait
+#pragma unroll
+        for (int q = 0; q < 16; q++) x[q] = q < p.parts ? w[q * (V + 2) + cc] : 0.f;
         float acc = 0.f;
-        for (int q = 0; q < p.parts; q++) {
-            const float e = __shfl(eq, q, 64);
-            if (c < V) acc = fmaf(e, w[q * (V + 2) + c], acc);
-        }
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc = fmaf(__shfl(eq, q, 64), x[q], acc);
         if (c < V) {
             const int64_t at = (int64_t)row * V + c;
             if (p.out_f32) ((float *)p.out)[at] = acc * g;
