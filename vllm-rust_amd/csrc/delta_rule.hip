@@ -38,8 +38,8 @@ struct ConvArgs {
 
 // one wave per (token, run of `group` channels); runs past the unit groups are plain 64-channel runs
 __global__ __launch_bounds__(256) void short_conv_silu_kernel(const ConvArgs a) {
-    const int t = blockIdx.y, lane = threadIdx.x & 63;
-    const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int t = blockIdx.x, lane = threadIdx.x & 63;   // tokens on x (no 65535 limit)
+    const int run = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int unit_ch = a.unit_groups * a.group;
     int c0, c1;
     bool unit = false;
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void short_conv_state_kernel(const ConvArgs a,
 __global__ __launch_bounds__(256) void delta_gates_kernel(float *__restrict__ g, int64_t ldg, const uint16_t *__restrict__ a_log,
                                                            const uint16_t *__restrict__ dt_bias, float *__restrict__ beta, int64_t ldbeta,
                                                            int heads, int dim) {
-    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c < heads * dim) {
         const float rate = expf(vmx_bf16_to_f32(a_log[c / dim]));
         const float dt = softplus_f(g[(int64_t)t * ldg + c] + vmx_bf16_to_f32(dt_bias[c]));
@@ -292,7 +292,7 @@ extern "C" int vmx_short_conv_silu(const float *x, int64_t ldx, const uint16_t *
     const ConvArgs a = conv_args(x, ldx, taps_bf16, state, y, ldy, positions, seq_ids, seq_starts, state_slots, tokens, channels, taps, unit_group,
                                  unit_groups, scaled_groups, unit_eps, scaled_mul);
     const int runs = unit_groups + (channels - unit_groups * unit_group + 63) / 64;
-    hipLaunchKernelGGL(short_conv_silu_kernel, dim3((runs + 3) / 4, tokens), dim3(256), 0, vmx_stream(stream), a);
+    hipLaunchKernelGGL(short_conv_silu_kernel, dim3(tokens, (runs + 3) / 4), dim3(256), 0, vmx_stream(stream), a);
     VMX_CHECK_LAUNCH("short_conv_silu");
     return VMX_OK;
 }
@@ -312,7 +312,7 @@ extern "C" int vmx_delta_rule_gates(float *g, int64_t ldg, const uint16_t *a_log
     VMX_REQUIRE(g && a_log_bf16 && dt_bias_bf16 && beta, "delta_rule_gates: null pointer");
     VMX_REQUIRE(heads >= 1 && dim >= 1 && ldg >= (int64_t)heads * dim && ldbeta >= heads, "delta_rule_gates: bad sizes");
     if (tokens <= 0) return VMX_OK;
-    hipLaunchKernelGGL(delta_gates_kernel, dim3((heads * dim + 255) / 256, tokens), dim3(256), 0, vmx_stream(stream), g, ldg, a_log_bf16,
+    hipLaunchKernelGGL(delta_gates_kernel, dim3(tokens, (heads * dim + 255) / 256), dim3(256), 0, vmx_stream(stream), g, ldg, a_log_bf16,
                        dt_bias_bf16, beta, ldbeta, heads, dim);
     VMX_CHECK_LAUNCH("delta_rule_gates");
     return VMX_OK;

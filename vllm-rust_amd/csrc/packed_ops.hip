@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void moe_combine_f32_kernel(float *__restrict_
                                                                const int32_t *__restrict__ inv, const float *__restrict__ w, int k,
                                                                const float *__restrict__ shared, const float *__restrict__ gate,
                                                                int64_t ldgate, int width) {
-    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;   // tokens on x (no 65535 limit)
     if (i >= width) return;
     float acc = 0.f;
     for (int s = 0; s < k; s++) acc = fmaf(w[(int64_t)t * k + s], y[(int64_t)inv[(int64_t)t * k + s] * width + i], acc);
@@ -132,8 +132,8 @@ __global__ __launch_bounds__(256) void embed_scaled_f32_kernel(float *__restrict
 // act[r, j] = silu(gu[r, j]) * gu[r, ff + j]: the gated activation between the two products of a feed-forward whose gate and up
 // projections were computed as one product
 __global__ __launch_bounds__(256) void glu_silu_kernel(void *__restrict__ act, int act_f32, const float *__restrict__ gu, int ff) {
-    const int64_t r = blockIdx.y;
-    const int j = blockIdx.x * 256 + threadIdx.x;
+    const int64_t r = blockIdx.x;             // rows on x: a prompt's (token, expert) pairs can pass the 65535 of the other axes
+    const int j = blockIdx.y * 256 + threadIdx.x;
     if (j >= ff) return;
     const float g = gu[r * 2 * ff + j], u = gu[r * 2 * ff + ff + j];
     const float v = g / (1.0f + expf(-g)) * u;
@@ -151,7 +151,7 @@ int vmx_embed_scaled_f32(float *x, const uint16_t *embed, const int32_t *tokens,
 
 int vmx_glu_silu_rows(void *act, int act_f32, const float *gu, int rows, int ff, hipStream_t st) {
     if (rows <= 0) return VMX_OK;
-    hipLaunchKernelGGL(glu_silu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, st, act, act_f32, gu, ff);
+    hipLaunchKernelGGL(glu_silu_kernel, dim3(rows, (ff + 255) / 256), dim3(256), 0, st, act, act_f32, gu, ff);
     VMX_CHECK_LAUNCH("glu silu");
     return VMX_OK;
 }
@@ -178,7 +178,7 @@ int vmx_moe_inverse(int32_t *inv, const int32_t *sorted, const int32_t *total, i
 
 int vmx_moe_combine_f32(float *x, const float *y, const int32_t *inv, const float *w, int k, const float *shared, const float *gate,
                         int64_t ldgate, int T, int width, hipStream_t st) {
-    hipLaunchKernelGGL(moe_combine_f32_kernel, dim3((width + 255) / 256, T), dim3(256), 0, st, x, y, inv, w, k, shared, gate, ldgate, width);
+    hipLaunchKernelGGL(moe_combine_f32_kernel, dim3(T, (width + 255) / 256), dim3(256), 0, st, x, y, inv, w, k, shared, gate, ldgate, width);
     VMX_CHECK_LAUNCH("moe combine");
     return VMX_OK;
 }

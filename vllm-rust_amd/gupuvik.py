@@ -15,6 +15,7 @@ import ctypes as C
 import dataclasses
 import json
 import math
+import re
 from pathlib import Path
 
 import numpy as np
@@ -282,6 +283,9 @@ class GupuvikForCausalLM:
                 dtype = f.info(lib.vmx_safetensors_find(f._h, name.encode()))[1]
                 if dtype != "BF16":
                     raise ValueError(f"{model_dir}: tensor `{name}` is {dtype}; Gupuvik checkpoints hold bf16")
+                m = re.fullmatch(r"l(\d+)\.rg2(\.b)?", name)
+                if m and int(m.group(1)) < len(self.spec.layers) and self.spec.layers[int(m.group(1))].mlp is None:
+                    continue                 # the gate of a feed-forward this layer does not have
                 self.load_tensor(name, ck.get(name))
         finally:
             ck.close()
