@@ -497,6 +497,63 @@ def test_other_sizes(gpu, case, dtype):
     assert rel_err(feed(eng, "b", toks, (20, 2, 1)), want) <= TOL[dtype]
 
 
+def random_spec(seed):
+    """A model drawn at random: layer order, head counts, sizes (half of them multiples of 8, which the matrix-core attention
+    takes), windows, kept tokens, caps, shared caches, filter lengths, ranks, feed-forward kinds."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *a: a[int(rng.integers(len(a)))]   # noqa: E731
+    size = lambda lo, hi: 8 * int(rng.integers(1, hi // 8 + 1)) if rng.random() < 0.5 else int(rng.integers(lo, hi + 1))   # noqa: E731
+
+    def ff():
+        kind = pick(None, "dense", "moe", "moe")
+        if kind == "dense":
+            return dict(mlp="dense", ff=int(rng.integers(4, 70)))
+        if kind == "moe":
+            e = int(rng.integers(1, 10))
+            return dict(mlp="moe", experts=e, top=int(rng.integers(1, e + 1)), expert_ff=int(rng.integers(4, 40)))
+        return dict(mlp=None)
+    layers, own = [], []
+    for i in range(int(rng.integers(2, 6))):
+        kv = pick(1, 2, 3)
+        heads = kv * pick(1, 2, 3, 4, 8)
+        if rng.random() < 0.5:
+            layers.append(delta_layer(heads=heads, kv_heads=kv, dim=size(3, 80), vdim=size(3, 72), conv=int(rng.integers(1, 6)),
+                                      decay_rank=int(rng.integers(1, 13)), gate_rank=int(rng.integers(1, 13)), **ff()))
+            continue
+        mask = dict(window=pick(0, int(rng.integers(1, 40))), keep_first=int(rng.integers(0, 7)), softcap=pick(0.0, 5.0, 20.0), scale=pick(0.1, 0.3, 1.0))
+        if own and rng.random() < 0.4:
+            src = own[int(rng.integers(len(own)))]
+            l = layers[src]
+            layers.append(attn_layer(heads=l.kv_heads * pick(1, 3, 4), kv_heads=l.kv_heads, dim=l.dim, vdim=l.vdim, kv_from=src, **mask, **ff()))
+        else:
+            layers.append(attn_layer(heads=heads, kv_heads=kv, dim=size(3, 72), vdim=size(3, 72), **mask, **ff()))
+            own.append(i)
+    return small_spec(layers=layers, width=pick(24, 40, 52, 64), vocab=int(rng.integers(20, 90)), embed_scale=pick(1.0, 2.0, 4.0), norm_eps=pick(1e-6, 1e-5))
+
+
+@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_configurations(gpu, seed, dtype):
+    """Two requests of unequal length start together and decode together, a third is fed in portions: against the oracle."""
+    vmx, torch = gpu
+    spec = random_spec(seed)
+    if dtype == "bfloat16":
+        spec = sure_routing(spec)
+    model, eng, w = build(spec, dtype, seed=seed, block_size=[1, 2, 4, 8, 16][seed % 5], num_blocks=400 if seed % 5 == 0 else 120)
+    a, b, c = tokens_for(spec, 62, seed), tokens_for(spec, 33, seed + 50), tokens_for(spec, 41, seed + 90)
+    wa, wb = oracle_logits(spec, w, a), oracle_logits(spec, w, b)
+    lg, _, _ = eng.step([("a", a[:47], list(range(47))), ("b", b[:18], list(range(18)))])
+    ga, gb = [lg[:47].cpu().numpy()], [lg[47:].cpu().numpy()]
+    for p in range(15):
+        lg, _, _ = eng.step([("b", [b[18 + p]], [0]), ("a", [a[47 + p]], [0])])
+        gb.append(lg[:1].cpu().numpy())
+        ga.append(lg[1:].cpu().numpy())
+    assert rel_err(np.concatenate(ga), wa) <= TOL[dtype] and rel_err(np.concatenate(gb), wb) <= TOL[dtype]
+    eng.finish("a")
+    assert rel_err(feed(eng, "c", c, (17, 5, 2, 1)), oracle_logits(spec, w, c)) <= TOL[dtype]
+    model.close()
+
+
 def test_long_prompt_whole_and_in_portions(gpu):
     """16 500 tokens with four experts per token: more (token, expert) pairs than one launch axis of 65 535 takes.  The whole prompt
     in one step gives the same last rows as portions of 4 096 (the plain oracle is too slow for this length and checks the first
