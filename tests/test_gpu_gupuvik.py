@@ -554,6 +554,30 @@ def test_random_configurations(gpu, seed, dtype):
     model.close()
 
 
+@pytest.mark.parametrize("seed", [100, 101, 102, 103])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_configurations_on_long_sequences(gpu, seed, dtype):
+    """The same kind of model with windows of up to 300 keys and 700 tokens: key tiles, key shares and staging rounds all
+    wrap several times; 620 tokens as a prompt next to a short request, then 80 decoded."""
+    import dataclasses
+    vmx, torch = gpu
+    spec = random_spec(seed)
+    spec = dataclasses.replace(spec, layers=[dataclasses.replace(l, window=8 * l.window, keep_first=4 * l.keep_first) if l.mixer == "attention" else l
+                                             for l in spec.layers])
+    if dtype == "bfloat16":
+        spec = sure_routing(spec)
+    model, eng, w = build(spec, dtype, seed=seed, block_size=16, num_blocks=64, max_tokens=700)
+    a, b = tokens_for(spec, 700, seed), tokens_for(spec, 30, seed + 1)
+    want = oracle_logits(spec, w, a)
+    lg, _, _ = eng.step([("b", b[:9], []), ("a", a[:620], list(range(620)))])
+    got = [lg.cpu().numpy()]
+    for p in range(80):
+        entries = [("a", [a[620 + p]], [0])] + ([("b", [b[9 + p]], [])] if 9 + p < len(b) else [])
+        got.append(eng.step(entries)[0].cpu().numpy())
+    assert rel_err(np.concatenate(got), want) <= TOL[dtype]
+    model.close()
+
+
 def test_long_prompt_whole_and_in_portions(gpu):
     """16 500 tokens with four experts per token: more (token, expert) pairs than one launch axis of 65 535 takes.  The whole prompt
     in one step gives the same last rows as portions of 4 096 (the plain oracle is too slow for this length and checks the first
